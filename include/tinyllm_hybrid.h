@@ -10,7 +10,13 @@
  *                      positions on the first rot_dims dimensions of each head (adjacent pairs), unit-RMS
  *                      normalisation of q and k after the rotation, a score scale, a "sink" (one is added to the
  *                      softmax denominator: a key of score 0 without a value), a sigmoid output gate.
- *                      Query/key width and value width of a head are independent.
+ *                      Query/key width and value width of a head are independent.  Further options: a weighted RMS
+ *                      norm over the WHOLE q (and k) projection before the rotation (qk_norm), rotation of the pairs
+ *                      (i, i + rot_dims/2) instead of neighbours (rot_half), frequencies rescaled by wavelength
+ *                      (rot_scaling_kind 1), scores mixed across query heads before the softmax (talk_dev), a learned
+ *                      sink logit per head (sink_dev), a chunked causal mask (chunk: a query sees the keys of its own
+ *                      run of `chunk` positions only), values blended with the values the first such layer computed for
+ *                      the same token (v_mix).
  *   TL_MIX_DELTA       gated delta rule: a [key_dim, value_dim] float32 state per head that decays, is corrected
  *                      towards the new value along the new key and is read with the query; q/k/v pass a short
  *                      causal depthwise convolution + SiLU first.  The state and the convolution's last inputs
@@ -33,10 +39,12 @@
  *                      layer has no latent projection of its own and reads the pages of that earlier layer.
  *
  * Block forms: parallel_block 1 is x += m (mixer(h) + ff(h)) with one norm; 0 is the sequential pre-norm block
- * x += ls1 * mixer(norm1 x); x += ls2 * ff(norm2 x) with optional per-channel scales ls1 / ls2.  Norms: RMS or
+ * x += ls1 * mixer(norm1 x); x += ls2 * ff(norm2 x) with optional per-channel scales ls1 / ls2; 2 is the block with the norm on
+ * the branch's OUTPUT, x += m norm1(mixer(x)); x += m norm2(ff(x)), whose sublayers read the stream itself.  Norms: RMS or
  * Dynamic Tanh (tanh(alpha x) w + b).  Feed-forward kinds: W_down act(W_up h), W_down (act(W_gate h) * W_up h), or a
- * mixture of experts (softmax router with a selection-only correction, groups of neighbouring experts, identity
- * experts, a gated shared expert).
+ * mixture of experts (softmax or sigmoid router with a selection-only correction, groups of neighbouring experts, identity
+ * experts, a shared expert with or without a scalar gate; experts W_down act(W_up h) or, with moe_gated, W_down (act(W_gate h) *
+ * W_up h); the router's weight on the expert's output or, with moe_scale_input, on its input).
  *
  * A contiguous range of layers may be repeated ("loop"): each pass has its own K/V pages / state slots, and is
  * entered through a [width, 2 width] projection of the running stream beside the embedding output plus a per-pass
@@ -69,6 +77,9 @@ enum { TL_MIX_ATTENTION = 0, TL_MIX_DELTA = 1, TL_MIX_LINREC = 2, TL_MIX_LATENT 
 enum { TL_REC_CHANNEL = 0, TL_REC_EXPGATE = 1 };
 enum { TL_NORM_RMS = 0, TL_NORM_DYT = 1 };
 enum { TL_FF_PLAIN = 0, TL_FF_GATED = 1, TL_FF_MOE = 2 };
+enum { TL_ROUTER_SOFTMAX = 0, TL_ROUTER_SIGMOID = 1 };
+enum { TL_BLOCK_SEQUENTIAL = 0, TL_BLOCK_PARALLEL = 1, TL_BLOCK_POSTNORM = 2 };
+enum { TL_VMIX_NONE = 0, TL_VMIX_FIRST = 1, TL_VMIX_BLEND = 2 };
 enum { TL_ACT_GELU_ERF = 0, TL_ACT_GELU_TANH = 1, TL_ACT_SILU = 2, TL_ACT_RELU2 = 3 };
 enum { TL_HY_F32 = 0, TL_HY_BF16 = 2 }; /* the values of tl_dtype in tinyllm_hip.h */
 
@@ -86,7 +97,9 @@ enum { TL_HY_F32 = 0, TL_HY_BF16 = 2 }; /* the values of tl_dtype in tinyllm_hip
  *   plain: up (ff)                   -> w_out2 [width, ff]
  *   gated: gate (ff) | up (ff)       -> w_out2 [width, ff]
  *   moe:   shared up (shared_ff) | expert 0 up (expert_ff) | expert 1 up ... | router (experts + identity) | shared gate (1) |
- *          zero rows up to a multiple of 8         -> w_out2 [width, shared_ff + experts * expert_ff]: shared down | expert 0 down | ... */
+ *          zero rows up to a multiple of 8         -> w_out2 [width, shared_ff + experts * expert_ff]: shared down | expert 0 down | ...
+ *   moe with moe_gated: shared gate (shared_ff) | expert 0 gate | ... | shared up (shared_ff) | expert 0 up | ... | router (experts + identity) |
+ *          [scalar shared gate (1) if moe_shared_sg] | zero rows up to a multiple of 8         -> w_out2 as above */
 typedef struct tl_hybrid_layer {
     int kind;
     int heads, kv_heads, dim, vdim;
@@ -133,13 +146,33 @@ typedef struct tl_hybrid_layer {
     const void *uk_t_dev;   /* [heads, kv_rank, dim]: W_uk of every head transposed */
     const void *uv_dev;     /* [heads, vdim, kv_rank] */
     float rot_factor, rot_original, rot_fast, rot_slow; /* rot_factor <= 0: plain frequencies */
+    /* attention, further options */
+    int qk_norm;            /* 1: q and k each pass an RMS norm over their whole projection (all heads at once) with the weights below,
+                               before the rotation */
+    const float *q_norm_dev, *k_norm_dev; /* [heads*dim], [kv_heads*dim] */
+    int rot_half;           /* 1: the rotation pairs dimension i with i + rot_dims/2; 0: 2i with 2i+1 */
+    int rot_scaling_kind;   /* 0: by dimension index (rot_fast / rot_slow = turns over rot_original positions, cos and sin grow);
+                               1: by wavelength l = 2 pi / f: f kept where l < rot_original / rot_fast, f / rot_factor where
+                               l > rot_original / rot_slow, blended linearly in original / l between */
+    const float *talk_dev;  /* [heads, heads]: score_h <- sum_g talk[h, g] score_g before the softmax; NULL: none */
+    const float *sink_dev;  /* [heads]: with sink != 0 the denominator gains exp(sink_dev[h]) instead of 1; NULL: 1 */
+    int chunk;              /* > 0: query i sees key j <= i only if i / chunk == j / chunk (positions of the sequence) */
+    int v_mix;              /* TL_VMIX_FIRST: this layer's values are kept for the step's rows; TL_VMIX_BLEND: v <- (1 - l) v + l v_first
+                               before they are cached */
+    float v_mix_lambda;
+    /* mixture of experts, further options */
+    int moe_router;         /* TL_ROUTER_*: scores softmax(z) or sigmoid(z) */
+    int moe_gated;          /* experts (and the shared one) are W_down (act(W_gate h) * W_up h) */
+    int moe_scale_input;    /* the router's weight multiplies the expert's input: expert(w h) */
+    int moe_shared_sg;      /* the shared expert is scaled by sigmoid of a scalar projection (its row follows the router's) */
 } tl_hybrid_layer;
 
 typedef struct tl_hybrid_config {
     int dtype;              /* TL_HY_BF16 or TL_HY_F32 */
     int width, vocab, num_layers;
     float norm_eps, residual_mult;
-    int parallel_block;     /* 1: x += m * (mixer(h) + ff(h)) with one norm; 0: x += m ls1 mixer(norm1 x), then x += m ls2 ff(norm2 x) */
+    int parallel_block;     /* TL_BLOCK_*: 1: x += m * (mixer(h) + ff(h)) with one norm; 0: x += m ls1 mixer(norm1 x), then x += m ls2 ff(norm2 x);
+                               2: x += m norm1(mixer(x)), then x += m norm2(ff(x)) */
     int loop_start, loop_stop, loop_times; /* loop_times <= 1 or start == stop: no loop */
     const void *loop_in_dev;    /* [width, 2*width], stream first */
     const float *loop_step_dev; /* [loop_times, width] */
@@ -152,6 +185,7 @@ typedef struct tl_hybrid_config {
     float final_norm_alpha;
     const float *final_norm_bias_dev;
     int page_size, num_pages, max_slots, max_pages_per_seq, max_rows;
+    float logit_scale;          /* logits = head . norm(x) * logit_scale (0 is read as 1) */
 } tl_hybrid_config;
 
 typedef struct tl_hybrid_stats {

@@ -474,3 +474,183 @@ def latent_layer(heads=4, dim=16, vdim=24, rot_dim=8, q_rank=20, kv_rank=40, bas
 
 def zefapel_config(layers, width=64, vocab=101, eps=1e-5, embed_scale=0.7):
     return {"architecture": "Zefapel", "embedding": {"scale": embed_scale}, "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+# ---- Lovulix: post-norm blocks x += norm1(mixer(x)); x += norm2(ff(x)) -------------------------------------------------------
+# mixer: grouped-query attention with an RMS norm over the WHOLE q (and k) projection, rotation of the pairs (i, i + dims/2) with
+# wavelength-dependent frequency rescaling, scores mixed across heads before the softmax, a chunked causal mask, a learned sink per
+# head in the denominator, values blended with the first such layer's values, a sigmoid output gate.
+# ff: experts chosen by the largest sigmoid(router) scores, the score multiplying the expert's INPUT, plus a shared expert.
+
+
+def wavelength_scaled_frequencies(dims, base, scaling=None):
+    """f_i = base^(-2i/dims), i < dims/2.  With ``scaling`` {factor, low, high, original}: by wavelength l = 2 pi / f, f stays where
+    l < original/high, becomes f / factor where l > original/low, and between the two is blended with s = (original/l - low) / (high - low):
+    (1 - s) f / factor + s f."""
+    f = np.array([base ** (-2.0 * i / dims) for i in range(dims // 2)])
+    if not scaling:
+        return f
+    out = f.copy()
+    fac, lo, hi, orig = scaling["factor"], scaling["low"], scaling["high"], scaling["original"]
+    for i, fi in enumerate(f):
+        l = 2.0 * math.pi / fi
+        if l < orig / hi:
+            continue
+        if l > orig / lo:
+            out[i] = fi / fac
+        else:
+            s = (orig / l - lo) / (hi - lo)
+            out[i] = (1.0 - s) * fi / fac + s * fi
+    return out
+
+
+def rotate_halves_by(z, positions, freqs):
+    """z [L, heads, dim]: with n = len(freqs), the pair (i, i + n) at position p turns by p * freqs[i]; dimensions from 2 n on pass."""
+    out = z.copy()
+    n = len(freqs)
+    for i, f in enumerate(freqs):
+        c, s = np.cos(positions * f)[:, None], np.sin(positions * f)[:, None]
+        u, v = z[..., i], z[..., i + n]
+        out[..., i] = u * c - v * s
+        out[..., i + n] = v * c + u * s
+    return out
+
+
+def talking_chunk_attention(q, k, v, scale, talk=None, sink=None, chunk=None):
+    """q [L, H, D], k [L, G, D], v [L, G, V].  Query i sees key j <= i of its own chunk (floor(i / chunk) == floor(j / chunk); chunk None:
+    every j <= i).  Scores q.k * scale of all heads are mixed per (i, j): s'_h = sum_g talk[h, g] s_g.  Weights exp(s'_h) / (exp(sink_h) + sum)
+    (sink None: no extra term).  Head h reads the values of K/V head h // (H / G).  Row by row."""
+    L, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((L, H, v.shape[2]))
+    for i in range(L):
+        lo = (i // chunk) * chunk if chunk else 0
+        s = np.stack([(k[lo:i + 1, h // (H // G)] @ q[i, h]) * scale for h in range(H)])  # [H, keys]
+        if talk is not None:
+            s = talk @ s
+        for h in range(H):
+            e = np.exp(s[h])
+            den = e.sum() + (math.exp(sink[h]) if sink is not None else 0.0)
+            out[i, h] = (e / den) @ v[lo:i + 1, h // (H // G)]
+    return out
+
+
+def sigmoid_top_route(z, top):
+    """Router logits z [E] -> {expert: weight}: the `top` largest sigmoid(z) (ties to the lower index), weight = the score itself."""
+    s = sigmoid(z)
+    return {j: s[j] for j in sorted(range(len(z)), key=lambda j: (-s[j], j))[:top]}
+
+
+def gated_expert(W, p, h):
+    return (silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
+
+
+def lovulix_feed_forward(mlp, W, p, h):
+    out = np.zeros_like(h)
+    zs = h @ W[p + "router"].T
+    for t in range(h.shape[0]):
+        for j, w in sigmoid_top_route(zs[t], mlp["router"]["top"]).items():
+            out[t] += gated_expert(W, p + f"e{j}.", w * h[t])
+    if mlp.get("shared"):
+        out = out + gated_expert(W, p + "shared.", h)
+    return out
+
+
+def lovulix_forward(config, W, tokens, streams=None):
+    """Logits [L, vocab] of a whole sequence; ``streams`` (a list) receives the residual stream after every layer."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps = config["norm"]["eps"]
+    L = len(tokens)
+    pos = np.arange(L, dtype=np.float64)
+    x = W["embed"][np.asarray(tokens)]
+    v_first = None
+    for i, spec in enumerate(config["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", spec["mixer"]
+        if spec["type"] != "attention":
+            raise ValueError(spec["type"])
+        H, G, D, V = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        q = rms_norm(x @ W[m + "q"].T, W[m + "q.norm"], eps).reshape(L, H, D)
+        k = rms_norm(x @ W[m + "k"].T, W[m + "k.norm"], eps).reshape(L, G, D)
+        v = (x @ W[m + "v"].T).reshape(L, G, V)
+        rot = mc.get("rot")
+        if rot and rot.get("dims", 0):
+            f = wavelength_scaled_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
+            q, k = rotate_halves_by(q, pos, f), rotate_halves_by(k, pos, f)
+        if mc.get("v_mix"):
+            if v_first is None:
+                v_first = v
+            else:
+                lam = float(W[m + "vmix"])
+                v = (1.0 - lam) * v + lam * v_first
+        mask = mc.get("mask") or {}
+        o = talking_chunk_attention(q, k, v, mc["scale"], W[m + "talk"], W[m + "sink"], mask.get("size")).reshape(L, H * V)
+        o = o * sigmoid(x @ W[m + "g"].T)
+        x = x + rms_norm(o @ W[m + "o"].T, W[p + "norm1"], eps)
+        if spec.get("mlp"):
+            x = x + rms_norm(lovulix_feed_forward(spec["mlp"], W, p + "mlp.", x), W[p + "norm2"], eps)
+        if streams is not None:
+            streams.append(x.copy())
+    return rms_norm(x, W["final.norm"], eps) @ W["head"].T * config["logit_scale"]
+
+
+def make_lovulix_weights(config, seed=0):
+    """Random bf16-representable weights by tensor name (float32 arrays) for a Lovulix config dict."""
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    Wd, out = config["width"], {}
+
+    def mat(rows, cols, scale=None):
+        s = scale if scale is not None else cols ** -0.5
+        return (torch.randn(rows, cols, generator=gen) * s).to(torch.bfloat16).float().numpy()
+
+    def vec(n, scale=0.1, shift=0.0):
+        return (torch.randn(n, generator=gen) * scale + shift).to(torch.bfloat16).float().numpy()
+
+    out["embed"], out["head"], out["final.norm"] = mat(config["vocab"], Wd, 1.0), mat(config["vocab"], Wd), vec(Wd, 0.1, 1.0)
+    for i, spec in enumerate(config["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", spec["mixer"]
+        H, G, D, V = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        out[p + "norm1"] = vec(Wd, 0.1, 1.0)
+        out[m + "q"], out[m + "k"], out[m + "v"] = mat(H * D, Wd), mat(G * D, Wd), mat(G * V, Wd)
+        out[m + "q.norm"], out[m + "k.norm"] = vec(H * D, 0.2, 1.0), vec(G * D, 0.2, 1.0)
+        out[m + "vmix"] = np.float32(vec(1, 0.1, 0.4)[0])
+        out[m + "talk"] = (np.eye(H, dtype=np.float32) + mat(H, H, 0.3)).astype(np.float32)
+        out[m + "talk"] = torch.from_numpy(out[m + "talk"]).to(torch.bfloat16).float().numpy()
+        out[m + "sink"] = vec(H, 1.0, 0.5)
+        out[m + "g"], out[m + "o"] = mat(H * V, Wd), mat(Wd, H * V)
+        mlp = spec.get("mlp")
+        if mlp:
+            f = p + "mlp."
+            out[p + "norm2"] = vec(Wd, 0.1, 1.0)
+            out[f + "router"] = mat(mlp["router"]["experts"], Wd, 2.0 * Wd ** -0.5)
+            names = [f"e{e}." for e in range(mlp["router"]["experts"])]
+            sizes = [mlp["expert"]["ff"]] * len(names)
+            if mlp.get("shared"):
+                names.append("shared.")
+                sizes.append(mlp["shared"]["ff"])
+            for name, n in zip(names, sizes):
+                out[f + name + "gate"], out[f + name + "up"], out[f + name + "down"] = mat(n, Wd), mat(n, Wd), mat(Wd, n)
+    return out
+
+
+def lovulix_moe(experts=6, top=2, ff=24, shared=40):
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+def lovulix_layer(heads=4, kv_heads=2, dim=16, vdim=24, rot_dims=8, base=5000.0, scaling=(8.0, 1.0, 4.0, 64), scale=0.3, chunk=16, v_mix=True,
+                  mlp="default"):
+    rot = {"base": base, "dims": rot_dims}
+    if scaling:
+        rot["scaling"] = {"factor": scaling[0], "low": scaling[1], "high": scaling[2], "original": scaling[3]}
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot": rot, "scale": scale, "v_mix": v_mix}
+    if chunk:
+        mixer["mask"] = {"size": chunk}
+    return {"type": "attention", "mixer": mixer, "mlp": lovulix_moe() if mlp == "default" else mlp}
+
+
+def lovulix_config(layers, width=64, vocab=101, eps=1e-5, logit_scale=0.7):
+    return {"architecture": "Lovulix", "layers": layers, "logit_scale": logit_scale, "norm": {"eps": eps}, "vocab": vocab, "width": width}

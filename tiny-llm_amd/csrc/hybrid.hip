@@ -75,6 +75,8 @@ struct tl_hybrid {
     float *part_acc = nullptr, *part_ml = nullptr;  // attention partials of split key ranges: [max_slots, heads, 64, vdim] / [..., 2]
     bool attn_rows_only = false;                    // TL_HYBRID_ATTN_ROWS=1: the one-wave-per-row attention everywhere (A/B twin of the tile kernel)
     float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *obuf = nullptr, *logits = nullptr;
+    float *y = nullptr;     // [R, width] a branch's result ahead of its norm (the block with the norm on the branch's output)
+    float *vref = nullptr;  // [R, G * vdim] the values of the step's rows in the first value-mixing layer
     void *h = nullptr, *cat = nullptr, *cat2 = nullptr, *hsel = nullptr;
     int ld_proj = 0, ld_cat = 0;
     int32_t *meta_dev = nullptr, *meta_host = nullptr;  // step metadata (host side pinned)
@@ -107,6 +109,7 @@ static int mixer_cols(const tl_hybrid_layer &L) {  // rows of w_in that belong t
 static int ff_in_cols(const tl_hybrid_layer &L) {  // rows of the feed-forward's input matrix
     if (L.ff <= 0) return 0;
     if (L.ff_kind == TL_FF_GATED) return 2 * L.ff;
+    if (L.ff_kind == TL_FF_MOE && L.moe_gated) return (2 * L.ff + L.experts + L.identity + (L.moe_shared_sg ? 1 : 0) + 7) / 8 * 8;
     if (L.ff_kind == TL_FF_MOE) return (L.shared_ff + L.experts * L.expert_ff + L.experts + L.identity + 1 + 7) / 8 * 8;
     return L.ff;
 }
@@ -322,6 +325,24 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
 }
 
+// attention whose scores are mixed across heads, whose mask is chunked or whose sinks are learned: every query head of a row in one workgroup
+template <typename D>
+static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, const Meta &m, const StepShape &sh, const float *gate,
+                          int ldg, void *out, int ldo) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    const int nw = std::min(16, L.heads);
+    const size_t lds = ((size_t)L.heads * L.dim + (size_t)L.heads * 64 + (size_t)nw * 64) * sizeof(float);
+    TL_REQUIRE(lds <= 160 * 1024, "hybrid attention: heads * dim too large for the head-mixing kernel");
+    auto kern = attn_talk_rows_kernel<D>;
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, dim3(sh.rows), dim3(64 * nw), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.row_seq, m.row_pos, m.seq_slot,
+                       e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.talk_dev, L.sink, L.sink_dev, L.chunk, gate,
+                       ldg, (S *)out, ldo);
+    TL_CHECK_LAUNCH("hybrid attention (mixed heads)");
+    return TL_OK;
+}
+
 static int launch_linrec(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
     const bool chan = L.rec_kind == TL_REC_CHANNEL;
     const int ones = chan ? 0 : 1, VE = L.vdim + ones;
@@ -381,11 +402,17 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
     const int rows = sh.rows, n_seqs = sh.n_seqs, H = L.heads, HV = L.heads * L.vdim;
     if (L.kind == TL_MIX_ATTENTION) {
         const int G = L.kv_heads;
-        hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot,
-                           e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
-                           L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+        if (L.qk_norm || L.rot_half || L.v_mix != TL_VMIX_NONE)  // (options of the row-wise preparation; create checked that it covers the layer)
+            hipLaunchKernelGGL((attn_prep_row_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
+                               c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.rot_half, L.qk_norm, L.q_norm_dev, L.k_norm_dev,
+                               c.norm_eps, H, G, L.dim, L.vdim, L.v_mix, L.v_mix_lambda, e->vref, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+        else
+            hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot,
+                               e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
+                               L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
         TL_CHECK_LAUNCH("hybrid attention prep");
         const float *gate = L.gated ? e->proj + (size_t)(H + G) * L.dim + (size_t)G * L.vdim : nullptr;
+        if (L.talk_dev || L.sink_dev || L.chunk > 0) return attention_talk<D>(e, L, run.kpool, run.vpool, m, sh, gate, ldp, e->cat, ldcat);
         return attention_core<D>(e, L, run.kpool, run.vpool, L.vdim, m, sh, gate, ldp, e->cat, ldcat);
     }
     if (L.kind == TL_MIX_LATENT) {
@@ -457,9 +484,18 @@ static int ff_act_t(tl_hybrid *e, const tl_hybrid_layer &L, int rows, int ldp, i
     using S = typename D::storage;
     hipStream_t st = e->stream;
     if (L.ff_kind == TL_FF_MOE) {
+        const dim3 grid(rows, rows >= 64 ? 1 : std::max(1, std::min(64, L.ff / 1024)));
+        if (L.moe_gated) {  // gates | ups | router | [scalar shared gate] | padding
+            const int ET = L.experts + L.identity, r0 = up0 + 2 * L.ff;
+            hipLaunchKernelGGL((moe_gated_act_kernel<D>), grid, dim3(256), 0, st, e->proj, ldp, r0, L.moe_shared_sg ? r0 + ET : -1, up0, up0 + L.ff, L.experts,
+                               L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw, L.moe_router,
+                               L.moe_scale_input, L.ff_act);
+            TL_CHECK_LAUNCH("hybrid moe route (gated experts)");
+            return TL_OK;
+        }
         const int ET = L.experts + L.identity, r0 = up0 + L.ff;  // shared up | expert ups | router | shared gate | padding
-        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows, rows >= 64 ? 1 : std::max(1, std::min(64, L.ff / 1024))), dim3(256), 0, st, e->proj, ldp, r0, r0 + ET, up0, up0 + L.shared_ff,
-                           L.experts, L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw);
+        hipLaunchKernelGGL((moe_route_act_kernel<D>), grid, dim3(256), 0, st, e->proj, ldp, r0, r0 + ET, up0, up0 + L.shared_ff,
+                           L.experts, L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw, L.moe_router);
         TL_CHECK_LAUNCH("hybrid moe route");
         return TL_OK;
     }
@@ -497,7 +533,7 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
         const tl_hybrid_layer &L = e->layers[run.layer];
         // the first norm of the run after this one, if it is a Dynamic Tanh that reads the stream as this run leaves it
         NormTail next_first;
-        if (!c.parallel_block && ri + 1 < e->runs.size() && !e->runs[ri + 1].enters_pass) {
+        if (c.parallel_block == TL_BLOCK_SEQUENTIAL && ri + 1 < e->runs.size() && !e->runs[ri + 1].enters_pass) {
             const tl_hybrid_layer &Nx = e->layers[e->runs[ri + 1].layer];
             if (Nx.norm_kind == TL_NORM_DYT) next_first = tail_for(Nx.norm_dev, Nx.norm_bias_dev, Nx.norm_alpha);
         }
@@ -506,10 +542,42 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             TL_CHECK_LAUNCH("hybrid pack2");
             HY_TRY(linear_t<D>(e->cat2, 2 * W, c.loop_in_dev, e->x, W, rows, W, 2 * W, 2, 1.f, c.loop_step_dev + (size_t)run.pass * W, 0, st));
         }
+        const int nmix = mixer_cols(L), HV = L.heads * L.vdim;
+        if (c.parallel_block == TL_BLOCK_POSTNORM) {
+            // x += m norm1(W_o mixer(x));  x += m norm2(ff(x)): the sublayers read the stream itself, the norm sits on what they return
+            const size_t n = (size_t)rows * W;
+            if (!h_ready) {
+                hipLaunchKernelGGL((cast_rows_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->x, (S *)e->h, n);
+                TL_CHECK_LAUNCH("hybrid stream cast");
+            }
+            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, 0, 1.f, nullptr, 0, st));
+            HY_TRY(mixer_t<D>(e, ri, m, sh, nmix, HV));
+            HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->y, W, rows, W, HV, 0, 1.f, nullptr, 0, st));
+            hipLaunchKernelGGL((postnorm_add_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, st, e->x, e->y, L.norm_dev, L.norm_offset, c.norm_eps,
+                               c.residual_mult, (S *)e->h, W);
+            TL_CHECK_LAUNCH("hybrid norm on the mixer's output");
+            if (L.ff > 0) {
+                const int nin2 = ff_in_cols(L);
+                HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
+                HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
+                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->y, W, rows, W, L.ff, 0, 1.f, nullptr, 0, st));
+                if (L.ff_kind == TL_FF_MOE && L.identity > 0) {  // identity experts return their input: weight * h joins the branch ahead of its norm
+                    hipLaunchKernelGGL((identity_axpy_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->y, (const S *)e->h, e->idw,
+                                       (const float *)nullptr, 1.f, W, rows);
+                    TL_CHECK_LAUNCH("hybrid identity experts");
+                }
+                hipLaunchKernelGGL((postnorm_add_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, st, e->x, e->y, L.norm2_dev, L.norm_offset, c.norm_eps,
+                                   c.residual_mult, (S *)e->h, W);
+                TL_CHECK_LAUNCH("hybrid norm on the feed-forward's output");
+            }
+            h_ready = true;
+            if (e->trace && e->trace_buf && rows <= c.max_rows)
+                HY_HIP(hipMemcpyAsync(e->trace_buf + ri * (size_t)c.max_rows * W, e->x, (size_t)rows * W * 4, hipMemcpyDeviceToDevice, st));
+            continue;
+        }
         if (!h_ready) HY_TRY(norm_t<D>(e, L.norm_kind, L.norm_dev, L.norm_bias_dev, L.norm_alpha, L.norm_offset, e->h, nullptr, rows));
         h_ready = false;
-        const int nmix = mixer_cols(L), HV = L.heads * L.vdim;
-        if (c.parallel_block) {
+        if (c.parallel_block == TL_BLOCK_PARALLEL) {
             const int nin = nmix + L.ff, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
             HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nin, rows, nin, W, 0, 1.f, nullptr, 0, st));
             HY_TRY(mixer_t<D>(e, ri, m, sh, nin, ldcat));
@@ -551,6 +619,11 @@ static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
     if (n_want <= 0) return TL_OK;
     HY_TRY(norm_t<D>(e, c.final_norm_kind, c.final_norm_dev, c.final_norm_bias_dev, c.final_norm_alpha, c.final_norm_offset, e->hsel, m.want_rows, n_want));
     HY_TRY(linear_t<D>(e->hsel, c.width, c.head_dev, e->logits, c.vocab, n_want, c.vocab, c.width, 0, 1.f, nullptr, 0, e->stream));
+    if (c.logit_scale != 0.f && c.logit_scale != 1.f) {
+        const size_t n = (size_t)n_want * c.vocab;
+        hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, e->stream, e->logits, c.logit_scale, n);
+        TL_CHECK_LAUNCH("hybrid logit scale");
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(n_want), dim3(1024), 0, e->stream, e->logits, c.vocab, e->argmax_dev, set_pending ? m.want_slot : (const int32_t *)nullptr,
                        e->pending_dev);
     TL_CHECK_LAUNCH("hybrid argmax");
@@ -614,7 +687,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     const tl_hybrid_config &c = *cfg;
     TL_REQUIRE(c.dtype == TL_HY_BF16 || c.dtype == TL_HY_F32, "hybrid_create: dtype must be bfloat16 or float32");
     TL_REQUIRE(c.width > 0 && c.vocab > 0 && c.num_layers > 0, "hybrid_create: width, vocab and num_layers must be positive");
-    TL_REQUIRE(c.parallel_block == 0 || c.parallel_block == 1, "hybrid_create: parallel_block is 0 (sequential) or 1 (parallel)");
+    TL_REQUIRE(c.parallel_block >= 0 && c.parallel_block <= 2, "hybrid_create: parallel_block is 0 (sequential), 1 (parallel) or 2 (norm on the branch's output)");
     TL_REQUIRE(c.final_norm_kind == TL_NORM_RMS || (c.final_norm_kind == TL_NORM_DYT && c.final_norm_bias_dev), "hybrid_create: final norm kind");
     TL_REQUIRE(c.page_size > 0 && c.num_pages > 0 && c.max_slots > 0 && c.max_pages_per_seq > 0 && c.max_rows > 0, "hybrid_create: pool sizes must be positive");
     TL_REQUIRE(c.embed_dev && c.final_norm_dev && c.head_dev, "hybrid_create: embed, final norm and head are required");
@@ -632,7 +705,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         HY_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
         e->owns_stream = true;
     }
-    int max_in = 0, max_cat = 0, max_q = 0, max_c = 0, max_hv = 0, max_gh = 1, max_da = 1, max_db = 1;
+    int max_in = 0, max_cat = 0, max_q = 0, max_c = 0, max_hv = 0, max_gh = 1, max_da = 1, max_db = 1, vmix_width = 0;
     for (int i = 0; i < c.num_layers; ++i) {
         const tl_hybrid_layer &L = e->layers[i];
         TL_REQUIRE(L.kind == TL_MIX_ATTENTION || L.kind == TL_MIX_DELTA || L.kind == TL_MIX_LINREC || L.kind == TL_MIX_LATENT, "hybrid_create: unknown mixer kind");
@@ -640,7 +713,9 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         TL_REQUIRE(L.dim > 0 && L.dim <= 1024 && L.vdim > 0 && L.vdim <= 512, "hybrid_create: head widths: dim 1..1024, vdim 1..512");
         TL_REQUIRE(L.w_in_dev && L.w_out_dev && L.norm_dev && L.ff >= 0, "hybrid_create: layer matrices and norm are required");
         TL_REQUIRE(L.norm_kind == TL_NORM_RMS || (L.norm_kind == TL_NORM_DYT && L.norm_bias_dev), "hybrid_create: norm kind (Dynamic Tanh needs its bias)");
-        if (c.parallel_block) {
+        if (c.parallel_block == TL_BLOCK_POSTNORM)
+            TL_REQUIRE(L.norm_kind == TL_NORM_RMS && !L.ls1_dev && !L.ls2_dev && !looped, "hybrid_create: the block with the norm on the branch's output takes RMS norms, no layer scale and no loop");
+        if (c.parallel_block == TL_BLOCK_PARALLEL) {
             TL_REQUIRE(L.ff_kind == TL_FF_PLAIN && !L.ls1_dev && !L.ls2_dev, "hybrid_create: the parallel block takes a plain feed-forward and no layer scale");
         } else if (L.ff > 0) {
             TL_REQUIRE(L.norm2_dev && L.w_in2_dev && L.w_out2_dev && (L.norm_kind != TL_NORM_DYT || L.norm2_bias_dev),
@@ -651,12 +726,26 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
                 TL_REQUIRE(L.experts >= 0 && L.identity >= 0 && ET >= 1 && ET <= 256, "hybrid_create: between 1 and 256 experts (identity experts included)");
                 TL_REQUIRE(L.groups >= 1 && ET % L.groups == 0 && L.keep >= 1 && L.keep <= L.groups, "hybrid_create: expert groups must divide the experts; 1 <= keep <= groups");
                 TL_REQUIRE(L.top >= 1 && L.top <= L.keep * (ET / L.groups), "hybrid_create: top exceeds the experts of the kept groups");
-                TL_REQUIRE(L.expert_ff >= 0 && L.shared_ff >= 0 && L.ff == L.shared_ff + L.experts * L.expert_ff && L.correction_dev,
-                           "hybrid_create: mixture of experts: ff = shared_ff + experts * expert_ff, correction required");
+                TL_REQUIRE(L.expert_ff >= 0 && L.shared_ff >= 0 && L.ff == L.shared_ff + L.experts * L.expert_ff,
+                           "hybrid_create: mixture of experts: ff = shared_ff + experts * expert_ff");
+                TL_REQUIRE(L.correction_dev || L.moe_router == TL_ROUTER_SIGMOID, "hybrid_create: a softmax router needs its correction vector");
+                TL_REQUIRE(L.moe_router == TL_ROUTER_SOFTMAX || L.moe_router == TL_ROUTER_SIGMOID, "hybrid_create: unknown router kind");
+                TL_REQUIRE(L.moe_gated || (!L.moe_scale_input && !L.moe_shared_sg), "hybrid_create: a weight on the expert's input needs gated experts");
             }
         }
         if (L.kind == TL_MIX_ATTENTION) {
             TL_REQUIRE(L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.dim, "hybrid_create: rot_dims must be even and at most dim");
+            TL_REQUIRE(!L.qk_norm || (L.q_norm_dev && L.k_norm_dev), "hybrid_create: a norm over the whole q / k projection needs its weights");
+            TL_REQUIRE(!(L.qk_unit_rms && (L.qk_norm || L.rot_half || L.v_mix != TL_VMIX_NONE)),
+                       "hybrid_create: unit-RMS heads after the rotation do not combine with the whole-projection norm, half-split rotation pairs or value mixing");
+            TL_REQUIRE(L.chunk >= 0 && L.v_mix >= TL_VMIX_NONE && L.v_mix <= TL_VMIX_BLEND, "hybrid_create: chunk >= 0, v_mix 0..2");
+            if (L.v_mix != TL_VMIX_NONE) {
+                if (vmix_width == 0) {
+                    TL_REQUIRE(L.v_mix == TL_VMIX_FIRST, "hybrid_create: the first value-mixing layer keeps its values (v_mix 1), later ones blend (v_mix 2)");
+                    vmix_width = L.kv_heads * L.vdim;
+                } else
+                    TL_REQUIRE(L.v_mix == TL_VMIX_BLEND && L.kv_heads * L.vdim == vmix_width, "hybrid_create: value-mixing layers share one values width");
+            }
         } else if (L.kind == TL_MIX_LINREC) {
             TL_REQUIRE(L.kv_heads == L.heads && L.out_norm_dev, "hybrid_create: a linear recurrence has one key head per head and an output norm weight");
             if (L.rec_kind == TL_REC_CHANNEL)
@@ -680,8 +769,9 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
             TL_REQUIRE(L.conv_taps >= 1 && L.conv_taps <= 64 && L.conv_dev && L.a_log_dev && L.dt_bias_dev && L.out_norm_dev,
                        "hybrid_create: a delta layer needs conv taps and weights, a_log, dt_bias and its output norm");
         }
-        max_in = std::max(max_in, c.parallel_block ? mixer_cols(L) + L.ff : std::max(mixer_cols(L), ff_in_cols(L)));
-        max_cat = std::max(max_cat, c.parallel_block ? L.heads * L.vdim + L.ff : std::max(L.heads * L.vdim, L.ff));
+        const bool par = c.parallel_block == TL_BLOCK_PARALLEL;
+        max_in = std::max(max_in, par ? mixer_cols(L) + L.ff : std::max(mixer_cols(L), ff_in_cols(L)));
+        max_cat = std::max(max_cat, par ? L.heads * L.vdim + L.ff : std::max(L.heads * L.vdim, L.ff));
         max_hv = std::max(max_hv, L.heads * (L.vdim + 1));
         max_gh = std::max(max_gh, L.heads);
         if (L.kind == TL_MIX_ATTENTION) max_q = std::max(max_q, L.heads * L.dim);
@@ -723,7 +813,20 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         const int half = std::max(1, L.rot_dims / 2);
         std::vector<float> f(half, 0.f);
         for (int k = 0; k < L.rot_dims / 2; ++k) f[k] = (float)std::pow((double)L.rot_base, -2.0 * k / (double)L.rot_dims);
-        if (L.rot_factor > 0.f && L.rot_dims > 0) {
+        if (L.rot_factor > 0.f && L.rot_dims > 0 && L.rot_scaling_kind == 1) {
+            // rescaled by wavelength l = 2 pi / f: kept below original / fast, slowed by `factor` above original / slow, blended in original / l between
+            const double two_pi = 6.283185307179586476925287, dims = L.rot_dims, orig = L.rot_original, hi = L.rot_fast, lo = L.rot_slow, fac = L.rot_factor;
+            for (int k = 0; k < L.rot_dims / 2; ++k) {
+                const double fk = std::pow((double)L.rot_base, -2.0 * k / dims), l = two_pi / fk;
+                double v = fk;
+                if (l > orig / lo) v = fk / fac;
+                else if (!(l < orig / hi)) {
+                    const double sm = (orig / l - lo) / (hi - lo);
+                    v = (1.0 - sm) * fk / fac + sm * fk;
+                }
+                f[k] = (float)v;
+            }
+        } else if (L.rot_factor > 0.f && L.rot_dims > 0) {
             // rescaled frequencies: where(t) = the dimension that turns t times over `original` positions; dimensions below where(fast) keep
             // their frequency, those above where(slow) are slowed by `factor`, a linear ramp between; cos and sin grow by 0.1 ln(factor) + 1
             const double two_pi = 6.283185307179586476925287, dims = L.rot_dims, lb = std::log((double)L.rot_base);
@@ -778,6 +881,8 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     e->ld_cat = (max_cat + 7) / 8 * 8;
     HY_TRY(dev_alloc(p, &e->x, (size_t)R * W));
     HY_TRY(dev_alloc(p, &e->x0, (size_t)R * W));
+    if (c.parallel_block == TL_BLOCK_POSTNORM) HY_TRY(dev_alloc(p, &e->y, (size_t)R * W));
+    if (vmix_width > 0) HY_TRY(dev_alloc(p, &e->vref, (size_t)R * vmix_width));
     HY_TRY(dev_alloc(p, &e->proj, (size_t)R * e->ld_proj));
     HY_TRY(dev_alloc(p, &e->qbuf, (size_t)R * std::max(1, max_q)));
     HY_TRY(dev_alloc(p, &e->f32a, (size_t)R * std::max(1, max_c)));

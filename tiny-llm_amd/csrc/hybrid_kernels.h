@@ -672,6 +672,173 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, c
     }
 }
 
+// ---- attention, step 1 (row form): one workgroup per row prepares q, k and v with the options the head-wise kernel above does not have ----
+// qk_norm: q (all heads) and k (all K/V heads) are each divided by the RMS of their WHOLE projection and multiplied by qw / kw, before the rotation.
+// Rotation of the first rot_dims dimensions of each head by pos * inv_freq[i]: pairs (i, i + rot_dims/2) with rot_half, (2i, 2i+1) without.
+// v_mix 1: the row's values are kept in vref [rows, G*vdim]; 2: v <- (1 - lambda) v + lambda vref before they go to their page.
+template <typename D>
+__global__ __launch_bounds__(256) void attn_prep_row_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
+                                                            const int32_t *block_table, int max_pages, int page_size, const float *inv_freq, int rot_dims,
+                                                            int rot_half, int qk_norm, const float *qw, const float *kw, float eps, int H, int G, int dim, int vdim,
+                                                            int v_mix, float lambda, float *vref, float *qbuf, typename D::storage *kpool,
+                                                            typename D::storage *vpool) {
+    __shared__ float red[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int pos = row_pos[t], slot = seq_slot[row_seq[t]];
+    const int page = block_table[(size_t)slot * max_pages + pos / page_size], in_page = pos % page_size;
+    const float *row = proj + (size_t)t * ldp;
+    const int nq = H * dim, nk = G * dim, nv = G * vdim;
+    float inv_q = 1.f, inv_k = 1.f;
+    if (qk_norm) {
+        float sq = 0.f, sk = 0.f;
+        for (int c = tid; c < nq; c += 256) sq += row[c] * row[c];
+        for (int c = tid; c < nk; c += 256) sk += row[nq + c] * row[nq + c];
+        sq = block_sum(sq, red);
+        sk = block_sum(sk, red);
+        inv_q = 1.f / sqrtf(sq / (float)nq + eps);
+        inv_k = 1.f / sqrtf(sk / (float)nk + eps);
+    }
+    const int half = rot_dims / 2;
+    for (int e = tid; e < nq + nk; e += 256) {
+        const bool is_q = e < nq;
+        const int he = is_q ? e : e - nq, hh = he / dim, c = he % dim;
+        const float *src = row + (is_q ? 0 : nq) + (size_t)hh * dim;
+        const float *w = qk_norm ? (is_q ? qw : kw) + (size_t)hh * dim : nullptr;
+        const float inv = is_q ? inv_q : inv_k;
+        float val = src[c] * inv * (w ? w[c] : 1.f);
+        if (c < rot_dims) {
+            int partner, fi;
+            bool first;
+            if (rot_half) first = c < half, partner = first ? c + half : c - half, fi = first ? c : c - half;
+            else first = (c & 1) == 0, partner = first ? c + 1 : c - 1, fi = c >> 1;
+            const float other = src[partner] * inv * (w ? w[partner] : 1.f);
+            float sn, cs;
+            sincosf((float)pos * inv_freq[fi], &sn, &cs);
+            val = first ? val * cs - other * sn : val * cs + other * sn;
+        }
+        if (is_q) qbuf[(size_t)t * nq + he] = val;
+        else kpool[(((size_t)page * G + hh) * page_size + in_page) * dim + c] = D::from_float(val);
+    }
+    for (int e = tid; e < nv; e += 256) {
+        float v = row[nq + nk + e];
+        if (v_mix == 1) vref[(size_t)t * nv + e] = v;
+        else if (v_mix == 2) v = (1.f - lambda) * v + lambda * vref[(size_t)t * nv + e];
+        vpool[(((size_t)page * G + e / vdim) * page_size + in_page) * vdim + e % vdim] = D::from_float(v);
+    }
+}
+
+// ---- attention, step 2 with scores mixed across heads (row form): one workgroup per row, a wave per mixed head ----------------------------
+// For every tile of 64 keys the waves first form the raw scores of ALL query heads (lane = key; head h reads K/V head h / (H/G)) in LDS; then wave
+// w mixes them for its head, s'_h = sum_g talk[h, g] s_g (talk NULL: s_h), and keeps a running maximum / sum / weighted value sum in float32.
+// chunk > 0: the keys start at the first position of the query's chunk.  sink: the running pair starts at (sinks[h] or 0, 1).
+// More heads than waves: the waves take the heads in passes and the raw scores are formed again per pass.
+template <typename D>
+__global__ __launch_bounds__(1024) void attn_talk_rows_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
+                                                              const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
+                                                              const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
+                                                              float scale, const float *talk, int sink, const float *sinks, int chunk, const float *gate,
+                                                              int ldg, typename D::storage *out, int ldo) {
+    extern __shared__ float smem[];
+    const int nw = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float *qs = smem;                 // [H][dim]
+    float *sc = qs + (size_t)H * dim; // [H][64] raw scores of the tile
+    float *ps = sc + (size_t)H * 64;  // [nw][64] weights of the tile, per wave
+    const int t = blockIdx.x;
+    const int pos = row_pos[t], slot = seq_slot[row_seq[t]], HG = H / G;
+    const int32_t *bt = block_table + (size_t)slot * max_pages;
+    const int lo = chunk > 0 ? (pos / chunk) * chunk : 0;
+    for (int c = threadIdx.x; c < H * dim; c += blockDim.x) qs[c] = qbuf[(size_t)t * H * dim + c];
+    __syncthreads();
+    for (int h0 = 0; h0 < H; h0 += nw) {
+        const int hm = h0 + wave;
+        const bool live = hm < H;
+        const int gm = live ? hm / HG : 0;
+        float m = sink ? (sinks && live ? sinks[hm] : 0.f) : -INFINITY, l = sink ? 1.f : 0.f;
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // vdim <= 512
+        for (int kb = lo; kb <= pos; kb += 64) {
+            const int j = kb + lane;
+            for (int h = wave; h < H; h += nw) {
+                float d = 0.f;
+                if (j <= pos) {
+                    const typename D::storage *kr = kpool + (((size_t)bt[j / page_size] * G + h / HG) * page_size + j % page_size) * dim;
+                    const float *q = qs + (size_t)h * dim;
+                    for (int c = 0; c < dim; ++c) d += q[c] * D::to_float(kr[c]);
+                }
+                sc[h * 64 + lane] = d * scale;
+            }
+            __syncthreads();
+            if (live) {
+                float s;
+                if (talk) {
+                    s = 0.f;
+                    for (int g = 0; g < H; ++g) s += talk[hm * H + g] * sc[g * 64 + lane];
+                } else s = sc[hm * 64 + lane];
+                if (j > pos) s = -INFINITY;
+                const float m_new = fmaxf(m, wave_max(s));
+                const float p = (j <= pos) ? expf(s - m_new) : 0.f;
+                const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+                l = l * corr + wave_sum(p);
+                m = m_new;
+                ps[wave * 64 + lane] = p;  // (read by this wave only: its lanes run in lockstep)
+                __builtin_amdgcn_wave_barrier();
+                const int cnt = min(64, pos - kb + 1);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] *= corr;
+                for (int jj = 0; jj < cnt; ++jj) {
+                    const int jg = kb + jj;
+                    const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + gm) * page_size + jg % page_size) * vdim;
+                    const float pj = ps[wave * 64 + jj];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int c = lane + i * 64;
+                        if (c < vdim) acc[i] += pj * D::to_float(vr[c]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (live) {
+            const float invl = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = lane + i * 64;
+                if (c < vdim) {
+                    float o = acc[i] * invl;
+                    if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + (size_t)hm * vdim + c]);
+                    out[(size_t)t * ldo + (size_t)hm * vdim + c] = D::from_float(o);
+                }
+            }
+        }
+    }
+}
+
+// ---- the block whose norm sits on the branch's output: x += mult * y / sqrt(mean y^2 + eps) * (offset + w); h = x as D rows (the next sublayer's input) ----
+template <typename D>
+__global__ void postnorm_add_kernel(float *x, const float *y, const float *w, float offset, float eps, float mult, typename D::storage *h, int width) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const float *src = y + (size_t)r * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) ss += src[c] * src[c];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = x[(size_t)r * width + c] + mult * (src[c] * inv * (offset + w[c]));
+        x[(size_t)r * width + c] = v;
+        h[(size_t)r * width + c] = D::from_float(v);
+    }
+}
+// float32 rows -> D rows (the input of a sublayer that reads the stream itself)
+template <typename D>
+__global__ void cast_rows_kernel(const float *x, typename D::storage *out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = D::from_float(x[i]);
+}
+__global__ void scale_kernel(float *x, float a, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] *= a;
+}
+
 // ---- feed-forward activation: cat[t, col0 + c] = act(proj[t, up0 + c]) ---------------------------------------------------
 template <typename D>
 __global__ void ff_act_kernel(const float *proj, int ldp, int up0, int ff, int kind, typename D::storage *out, int ldo, int col0, int rows) {
@@ -1190,16 +1357,12 @@ __global__ __launch_bounds__(64) void linrec_out_kernel(const float *obuf, int V
 // group scores its largest choice, only the `keep` best groups can be taken; the `top` largest choices among them are taken (ties: the lower
 // index); weights are their s, not renormalised.  The last `identity` experts return their input: their weights are summed into idw[t].
 // cat row: [ sigmoid(sg) * relu(up)^2  (ffs) | w_e * relu(up_e)^2 (ffe each; 0 for experts not taken) ].
-template <typename D>
-__global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, int ldp, int r0, int sg0, int su0, int eu0, int experts, int identity, int top,
-                                                            int groups, int keep, int ffe, int ffs, const float *correction,
-                                                            typename D::storage *out, int ldo, int col0, float *idw) {
-    __shared__ float sw[256], sc[256];
-    __shared__ float gm[256];
-    // blockIdx.y: a share of the row's columns (every share routes the row again: a few dozen comparisons against thousands of columns)
-    const int t = blockIdx.x, tid = threadIdx.x, ET = experts + identity;
-    const float *row = proj + (size_t)t * ldp;
-    if (tid < 64) {  // one wave routes (ET <= 256: four experts a lane at most)
+// the router of one row, by every thread of a 256-thread workgroup: scores s = softmax(z) or sigmoid(z) (router 0 / 1); choice = s + correction
+// (NULL: 0); groups, kept groups, the `top` largest choices (ties: the lower index).  Leaves sw[e] = s_e for the experts taken, 0 for the others.
+__device__ __forceinline__ void moe_route_row(const float *row, int r0, int ET, int top, int groups, int keep, const float *correction, int router, float *sw,
+                                              float *sc, float *gm) {
+    const int tid = threadIdx.x;
+    if (tid < 64) {  // one wave scores (ET <= 256: four experts a lane at most)
         float z[4], mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -1207,26 +1370,32 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
             z[i] = e < ET ? row[r0 + e] : -INFINITY;
             mx = fmaxf(mx, z[i]);
         }
-        mx = wave_max(mx);
-        float sum = 0.f;
+        float sum = 1.f;
+        if (router == 0) {
+            mx = wave_max(mx);
+            sum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            z[i] = (tid + 64 * i) < ET ? expf(z[i] - mx) : 0.f;
-            sum += z[i];
+            for (int i = 0; i < 4; ++i) {
+                z[i] = (tid + 64 * i) < ET ? expf(z[i] - mx) : 0.f;
+                sum += z[i];
+            }
+            sum = wave_sum(sum);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) z[i] = (tid + 64 * i) < ET ? sigmoid_f(z[i]) : 0.f;
         }
-        sum = wave_sum(sum);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int e = tid + 64 * i;
             if (e < ET) {
-                const float s = z[i] / sum;
+                const float s = router == 0 ? z[i] / sum : z[i];
                 sw[e] = s;
-                sc[e] = s + correction[e];
+                sc[e] = s + (correction ? correction[e] : 0.f);
             }
         }
     }
     __syncthreads();
-    if (tid == 0) {  // groups, then the top choices: a few dozen comparisons
+    if (tid == 0 && groups > 1) {  // groups, then the top choices: a few dozen comparisons
         const int per = ET / groups;
         for (int g = 0; g < groups; ++g) {
             float m = -INFINITY;
@@ -1251,6 +1420,18 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
     __syncthreads();
     if (tid < ET) sw[tid] = wgt;
     __syncthreads();
+}
+
+template <typename D>
+__global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, int ldp, int r0, int sg0, int su0, int eu0, int experts, int identity, int top,
+                                                            int groups, int keep, int ffe, int ffs, const float *correction,
+                                                            typename D::storage *out, int ldo, int col0, float *idw, int router) {
+    __shared__ float sw[256], sc[256];
+    __shared__ float gm[256];
+    // blockIdx.y: a share of the row's columns (every share routes the row again: a few dozen comparisons against thousands of columns)
+    const int t = blockIdx.x, tid = threadIdx.x, ET = experts + identity;
+    const float *row = proj + (size_t)t * ldp;
+    moe_route_row(row, r0, ET, top, groups, keep, correction, router, sw, sc, gm);
     if (tid == 0 && blockIdx.y == 0) {
         float a = 0.f;
         for (int e = experts; e < ET; ++e) a += sw[e];
@@ -1262,6 +1443,38 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
     for (int c = blockIdx.y * per + tid; c < c_end; c += 256) {  // shared columns first, then the experts' (su0 + ffs == eu0)
         const float w = c < ffs ? sgate : sw[(c - ffs) / ffe], u = fmaxf(row[su0 + c], 0.f);
         o[c] = D::from_float(w * u * u);
+    }
+}
+// the same with gated experts, W_down (act(W_gate h) * W_up h): proj columns g0 .. = shared gate [ffs] | expert gates [ffe each], u0 .. = shared up | expert ups,
+// router logits at r0, the shared expert's scalar gate at sg0 (sg0 < 0: the shared expert is not scaled).  The router's weight w_e multiplies the
+// expert's OUTPUT (scale_input 0: w act(g) u) or its INPUT (1: the expert of w h, i.e. act(w g) (w u), both projections being linear).
+// cat row: [ shared (ffs) | expert columns (ffe each; 0 for experts not taken) ].
+template <typename D>
+__global__ __launch_bounds__(256) void moe_gated_act_kernel(const float *proj, int ldp, int r0, int sg0, int g0, int u0, int experts, int identity, int top,
+                                                            int groups, int keep, int ffe, int ffs, const float *correction, typename D::storage *out,
+                                                            int ldo, int col0, float *idw, int router, int scale_input, int act) {
+    __shared__ float sw[256], sc[256];
+    __shared__ float gm[256];
+    const int t = blockIdx.x, tid = threadIdx.x, ET = experts + identity;
+    const float *row = proj + (size_t)t * ldp;
+    moe_route_row(row, r0, ET, top, groups, keep, correction, router, sw, sc, gm);
+    if (tid == 0 && blockIdx.y == 0) {
+        float a = 0.f;
+        for (int e = experts; e < ET; ++e) a += sw[e];
+        idw[t] = a;
+    }
+    const float sgate = sg0 >= 0 ? sigmoid_f(row[sg0]) : 1.f;
+    typename D::storage *o = out + (size_t)t * ldo + col0;
+    const int n = ffs + experts * ffe, per = (n + gridDim.y - 1) / gridDim.y, c_end = min(n, (int)(blockIdx.y + 1) * per);
+    for (int c = blockIdx.y * per + tid; c < c_end; c += 256) {
+        const float g = row[g0 + c], u = row[u0 + c];
+        float v;
+        if (c < ffs) v = sgate * act_f(g, act) * u;
+        else {
+            const float w = sw[(c - ffs) / ffe];
+            v = w == 0.f ? 0.f : (scale_input ? act_f(w * g, act) * (w * u) : w * act_f(g, act) * u);
+        }
+        o[c] = D::from_float(v);
     }
 }
 // identity experts: x[t, c] += ls[c] * idw[t] * h[t, c]  (ls may be null: 1)

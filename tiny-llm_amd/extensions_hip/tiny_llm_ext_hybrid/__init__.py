@@ -26,6 +26,9 @@ MIX_ATTENTION, MIX_DELTA, MIX_LINREC, MIX_LATENT = 0, 1, 2, 3
 REC_CHANNEL, REC_EXPGATE = 0, 1
 NORM_RMS, NORM_DYT = 0, 1
 FF_PLAIN, FF_GATED, FF_MOE = 0, 1, 2
+ROUTER_SOFTMAX, ROUTER_SIGMOID = 0, 1
+BLOCK_SEQUENTIAL, BLOCK_PARALLEL, BLOCK_POSTNORM = 0, 1, 2
+VMIX_NONE, VMIX_FIRST, VMIX_BLEND = 0, 1, 2
 HY_F32, HY_BF16 = 0, 2
 FF_GELU_ERF, FF_GELU_TANH, FF_SILU, FF_RELU2 = 0, 1, 2, 3
 
@@ -44,7 +47,10 @@ class TlHybridLayer(ctypes.Structure):
                 ("i_bias_dev", _vp), ("f_bias_dev", _vp),
                 ("q_rank", _i), ("kv_rank", _i), ("rot_dim", _i), ("kv_from", _i), ("dq_norm_dev", _vp), ("dkv_norm_dev", _vp),
                 ("uq_dev", _vp), ("uk_t_dev", _vp), ("uv_dev", _vp),
-                ("rot_factor", _f), ("rot_original", _f), ("rot_fast", _f), ("rot_slow", _f)]
+                ("rot_factor", _f), ("rot_original", _f), ("rot_fast", _f), ("rot_slow", _f),
+                ("qk_norm", _i), ("q_norm_dev", _vp), ("k_norm_dev", _vp), ("rot_half", _i), ("rot_scaling_kind", _i),
+                ("talk_dev", _vp), ("sink_dev", _vp), ("chunk", _i), ("v_mix", _i), ("v_mix_lambda", _f),
+                ("moe_router", _i), ("moe_gated", _i), ("moe_scale_input", _i), ("moe_shared_sg", _i)]
 
 
 class TlHybridConfig(ctypes.Structure):
@@ -53,7 +59,8 @@ class TlHybridConfig(ctypes.Structure):
                 ("loop_in_dev", _vp), ("loop_step_dev", _vp), ("embed_dev", _vp), ("final_norm_dev", _vp),
                 ("final_norm_offset", _f), ("head_dev", _vp),
                 ("embed_scale", _f), ("final_norm_kind", _i), ("final_norm_alpha", _f), ("final_norm_bias_dev", _vp),
-                ("page_size", _i), ("num_pages", _i), ("max_slots", _i), ("max_pages_per_seq", _i), ("max_rows", _i)]
+                ("page_size", _i), ("num_pages", _i), ("max_slots", _i), ("max_pages_per_seq", _i), ("max_rows", _i),
+                ("logit_scale", _f)]
 
 
 class TlHybridStats(ctypes.Structure):

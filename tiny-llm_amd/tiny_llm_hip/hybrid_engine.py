@@ -23,6 +23,9 @@ _MIX = {"attention": 0, "delta": 1, "linrec": 2, "latent": 3}
 _REC = {"channel": 0, "expgate": 1}
 _NORM = {"rms": 0, "dyt": 1}
 _FF_KIND = {"plain": 0, "gated": 1, "moe": 2}
+_BLOCK = {"sequential": 0, "parallel": 1, "postnorm": 2}
+_VMIX = {"none": 0, "first": 1, "blend": 2}
+_ROUTER = {"softmax": 0, "sigmoid": 1}
 
 
 class HybridEngine:
@@ -73,6 +76,15 @@ class HybridEngine:
             s.ff_kind, s.experts, s.identity, s.top, s.groups, s.keep = _FF_KIND[L.ff_kind], L.experts, L.identity, L.top, L.groups, L.keep
             s.expert_ff, s.shared_ff, s.correction_dev = L.expert_ff, L.shared_ff, ptr("correction")
             s.kv_from = -1
+            s.moe_router, s.moe_gated, s.moe_scale_input = _ROUTER[L.router], int(L.moe_gated), int(L.moe_scale_input)
+            s.moe_shared_sg = int(L.moe_gated and L.moe_shared_sg)
+            if L.kind == "attention":
+                s.qk_norm, s.q_norm_dev, s.k_norm_dev, s.rot_half = int(L.qk_norm), ptr("q_norm"), ptr("k_norm"), int(L.rot_half)
+                s.talk_dev, s.sink_dev, s.chunk = ptr("talk"), ptr("sink"), L.chunk
+                s.v_mix, s.v_mix_lambda = _VMIX[L.v_mix], t.get("v_mix_lambda", 0.0)
+                if L.rot_scaling:
+                    s.rot_factor, s.rot_original, s.rot_fast, s.rot_slow = L.rot_scaling
+                    s.rot_scaling_kind = 1 if L.rot_scaling_kind == "wavelength" else 0
             if L.kind == "linrec":
                 s.rec_kind, s.gate_cap, s.tau, s.a_rank, s.out_norm_dev = _REC[L.rec_kind], L.gate_cap, L.tau, max(L.a_rank, 0), t["out_norm"].data_ptr()
                 s.a2_dev, s.a2_bias_dev, s.i_bias_dev, s.f_bias_dev = ptr("a2"), ptr("a2_bias"), ptr("i_bias"), ptr("f_bias")
@@ -84,7 +96,7 @@ class HybridEngine:
         c = ext.TlHybridConfig()
         c.dtype = ext.HY_BF16 if dtype == torch.bfloat16 else ext.HY_F32
         c.width, c.vocab, c.num_layers, c.norm_eps, c.residual_mult = cfg.width, cfg.vocab, len(cfg.layers), cfg.norm_eps, cfg.residual_mult
-        c.parallel_block, c.embed_scale = int(cfg.block == "parallel"), cfg.embed_scale
+        c.parallel_block, c.embed_scale, c.logit_scale = _BLOCK[cfg.block], cfg.embed_scale, cfg.logit_scale
         c.final_norm_kind, c.final_norm_alpha = _NORM[cfg.norm_kind], w.get("final_norm_alpha", 0.0)
         c.final_norm_bias_dev = w["final_norm_bias"].data_ptr() if "final_norm_bias" in w else None
         if cfg.loop:

@@ -41,6 +41,19 @@ per-channel layer scales ls1 / ls2:
     ff "moe": s = softmax(W_router h) over experts + identity experts; choice = s + correction; experts form groups.count runs of
         neighbours, the groups.keep groups with the largest choice stay; the `top` largest choices among them are taken with weight s
         (not renormalised); expert = W_down relu(W_up h)^2, identity expert = h; plus sigmoid(W_sg h) * shared expert.
+
+Lovulix -- x = embed[token]; per layer the norm sits on what a branch RETURNS and the branches read the stream itself:
+
+    x <- x + norm1(mixer(x));   x <- x + norm2(ff(x))          norm: y / sqrt(mean y^2 + eps) * w;  logits = head norm(x) * logit_scale
+
+    mixer "attention": grouped-query attention.  q and k each pass an RMS norm over their whole projection (all heads at once, weights
+        q.norm / k.norm); the first rot.dims dimensions of each head turn as pairs (i, i + dims/2) by p * f_i, f_i = base^(-2i/dims) rescaled by
+        wavelength l = 2 pi / f (rot.scaling: kept where l < original/high, f / factor where l > original/low, blended linearly in
+        original / l between); scores q.k * scale are mixed across heads, s_h <- sum_g talk[h, g] s_g; query i sees key j <= i of its own run of
+        mask.size positions; weights exp(s_h) / (exp(sink_h) + sum exp); with v_mix every such layer but the first caches
+        v <- (1 - vmix) v + vmix v_first (the first such layer's values of the same token); heads * sigmoid(W_g x); W_o.
+    ff "moe": s = sigmoid(W_router x); the `top` largest s are taken; each contributes expert(s_e x) -- the score scales the expert's INPUT --
+        with expert(u) = W_down (silu(W_gate u) * W_up u); plus a shared expert of the same form on x.
 """
 
 from __future__ import annotations
@@ -50,7 +63,7 @@ from typing import Any, Callable
 
 import torch
 
-__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "zefapel_config", "pack_layer_list"]
+__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "zefapel_config", "lovulix_config", "pack_layer_list"]
 
 
 @dataclass
@@ -92,6 +105,20 @@ class LayerSpec:
     rot_dim: int = 0
     kv_from: int = -1               # layer whose latent cache is read; -1: the layer's own
     rot_scaling: tuple[float, float, float, float] | None = None  # (factor, original, fast, slow)
+    # attention, further options
+    qk_norm: bool = False           # weighted RMS norm over the whole q / k projection before the rotation (tensors mix.q.norm / mix.k.norm)
+    rot_half: bool = False          # rotation pairs (i, i + rot_dims/2) instead of (2i, 2i+1)
+    rot_scaling_kind: str = "index" # "index": rot_scaling by dimension index | "wavelength": (factor, original, high, low) by wavelength
+    talk: bool = False              # scores mixed across heads before the softmax (tensor mix.talk [heads, heads])
+    learned_sink: bool = False      # the sink's logit is a tensor (mix.sink [heads]) instead of 0
+    chunk: int = 0                  # > 0: chunked causal mask
+    v_mix: str = "none"             # "first": keeps its values for later layers | "blend": v <- (1 - l) v + l v_first (tensor mix.vmix)
+    # mixture of experts, further options
+    router: str = "softmax"         # "softmax" | "sigmoid"
+    moe_gated: bool = False         # experts W_down (act(W_gate h) * W_up h)
+    moe_scale_input: bool = False   # the router's weight multiplies the expert's input
+    moe_shared_sg: bool = True      # the shared expert is scaled by sigmoid of a scalar projection
+    moe_correction: bool = True     # a selection-only correction vector (tensor mlp.correction)
 
 
 @dataclass
@@ -106,8 +133,10 @@ class LayerListConfig:
     loop: tuple[int, int, int] | None = None  # (start, stop, times)
     norm_kind: str = "rms"          # "rms" | "dyt" (tanh(alpha x) w + b: tensors <name>, <name>.alpha, <name>.b)
     block: str = "parallel"         # "parallel": x += m (mixer(h) + ff(h)), one norm | "sequential": two norms, two residual sums
+                                    # | "postnorm": x += m norm1(mixer(x)); x += m norm2(ff(x))
     layer_scale: bool = False       # sequential block: per-channel vectors ls1 / ls2 on the branches
     embed_scale: float = 1.0
+    logit_scale: float = 1.0
     prefix: Callable[[int], str] = field(default=lambda i: f"l{i}.")
 
     @property
@@ -223,6 +252,63 @@ def zefapel_config(config: dict) -> LayerListConfig:
                            embed_scale=float(config["embedding"]["scale"]))
 
 
+def lovulix_config(config: dict) -> LayerListConfig:
+    """config.json of a Lovulix checkpoint -> LayerListConfig.  Every size and every constant the file gives is read from it."""
+    for key in ("layers", "norm", "logit_scale", "vocab", "width"):
+        if key not in config:
+            raise ValueError(f"config.json lacks {key!r}")
+    layers, first_mix = [], True
+    for i, entry in enumerate(config["layers"]):
+        kind, mc, mlp = entry.get("type"), entry.get("mixer") or {}, entry.get("mlp")
+        if kind != "attention":
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        ff: dict[str, Any] = {}
+        if mlp is not None:
+            if mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: unsupported mlp.kind={mlp.get('kind')!r}")
+            r, shared = mlp["router"], mlp.get("shared")
+            experts, expert_ff = int(r["experts"]), int(mlp["expert"]["ff"])
+            shared_ff = int(shared["ff"]) if shared else 0
+            if not 1 <= int(r["top"]) <= experts:
+                raise ValueError(f"layer {i}: top={r['top']} of {experts} experts")
+            ff = dict(ff=shared_ff + experts * expert_ff, ff_kind="moe", ff_act="silu", experts=experts, top=int(r["top"]), expert_ff=expert_ff,
+                      shared_ff=shared_ff, router="sigmoid", moe_gated=True, moe_scale_input=True, moe_shared_sg=False, moe_correction=False)
+        rot, sc = mc.get("rot") or {}, None
+        if rot.get("scaling"):
+            g = rot["scaling"]
+            sc = (float(g["factor"]), float(g["original"]), float(g["high"]), float(g["low"]))
+        v_mix = "none"
+        if mc.get("v_mix"):
+            v_mix, first_mix = ("first" if first_mix else "blend"), False
+        mask = mc.get("mask") or {}
+        layers.append(LayerSpec(kind="attention", heads=int(mc["heads"]), kv_heads=int(mc["kv_heads"]), dim=int(mc["dim"]), vdim=int(mc["vdim"]),
+                                rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), rot_scaling=sc, rot_scaling_kind="wavelength",
+                                rot_half=True, scale=float(mc["scale"]), qk_norm=True, sink=True, learned_sink=True, talk=True, gated=True,
+                                chunk=int(mask.get("size", 0)), v_mix=v_mix, **ff))
+    return LayerListConfig(family="Lovulix", width=int(config["width"]), vocab=int(config["vocab"]), norm_eps=float(config["norm"]["eps"]),
+                           residual_mult=1.0, layers=layers, norm_offset=0.0, block="postnorm", logit_scale=float(config["logit_scale"]))
+
+
+def _lovulix_tensor_shapes(cfg: LayerListConfig) -> dict[str, tuple[int, ...]]:
+    """Every tensor a Lovulix checkpoint must hold, with its shape."""
+    W = cfg.width
+    want: dict[str, tuple[int, ...]] = {"embed": (cfg.vocab, W), "final.norm": (W,), "head": (cfg.vocab, W)}
+    for i, L in enumerate(cfg.layers):
+        p, m = cfg.prefix(i), cfg.prefix(i) + "mix."
+        hv = L.heads * L.vdim
+        want.update({p + "norm1": (W,), m + "q": (L.heads * L.dim, W), m + "k": (L.kv_heads * L.dim, W), m + "v": (L.kv_heads * L.vdim, W),
+                     m + "q.norm": (L.heads * L.dim,), m + "k.norm": (L.kv_heads * L.dim,), m + "talk": (L.heads, L.heads), m + "sink": (L.heads,),
+                     m + "g": (hv, W), m + "o": (W, hv)})
+        if L.v_mix == "blend":  # (the first value-mixing layer's scalar is not read)
+            want[m + "vmix"] = ()
+        if L.ff:
+            f = p + "mlp."
+            want.update({p + "norm2": (W,), f + "router": (L.experts, W)})
+            for name, n in [(f"e{e}.", L.expert_ff) for e in range(L.experts)] + ([("shared.", L.shared_ff)] if L.shared_ff else []):
+                want.update({f + name + "gate": (n, W), f + name + "up": (n, W), f + name + "down": (W, n)})
+    return want
+
+
 def _norm_shapes(cfg: LayerListConfig, name: str) -> dict[str, tuple[int, ...]]:
     if cfg.norm_kind == "dyt":
         return {name: (cfg.width,), name + ".b": (cfg.width,), name + ".alpha": ()}
@@ -269,6 +355,7 @@ def _zefapel_tensor_shapes(cfg: LayerListConfig) -> dict[str, Any]:
 FAMILIES: dict[str, tuple[Callable[[dict], LayerListConfig], Callable[[LayerListConfig], dict]]] = {
     "Fonapel": (fonapel_config, _fonapel_tensor_shapes),
     "Zefapel": (zefapel_config, _zefapel_tensor_shapes),
+    "Lovulix": (lovulix_config, _lovulix_tensor_shapes),
 }
 
 
@@ -309,6 +396,15 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
             rows = [mat(p + "mix.q"), mat(p + "mix.k"), mat(p + "mix.v")]
             if L.kind != "attention" or L.gated:
                 rows.append(mat(p + "mix.g"))
+        if L.kind == "attention":
+            if L.qk_norm:
+                entry["q_norm"], entry["k_norm"] = vec(p + "mix.q.norm"), vec(p + "mix.k.norm")
+            if L.talk:
+                entry["talk"] = vec(p + "mix.talk")
+            if L.learned_sink:
+                entry["sink"] = vec(p + "mix.sink")
+            if L.v_mix == "blend":
+                entry["v_mix_lambda"] = float(tensors[p + "mix.vmix"].float())
         if L.kind == "delta":
             rows += [mat(p + "mix.a"), mat(p + "mix.b")]
             entry["conv"] = torch.cat([vec(p + "mix.q.conv"), vec(p + "mix.k.conv"), vec(p + "mix.v.conv")], 0).contiguous()
@@ -328,6 +424,19 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
                 ff_rows, ff_out = [mat(f + "up")], [mat(f + "down")]
             elif L.ff_kind == "gated":
                 ff_rows, ff_out = [mat(f + "gate"), mat(f + "up")], [mat(f + "down")]
+            elif L.moe_gated:
+                # gates (shared | experts) | ups (shared | experts) | router | [scalar shared gate] | zero rows up to a multiple of 8
+                W = cfg.width
+                names = (["shared."] if L.shared_ff else []) + [f"e{e}." for e in range(L.experts)]
+                ff_rows = [mat(f + n + "gate") for n in names] + [mat(f + n + "up") for n in names] + [mat(f + "router")]
+                if L.moe_shared_sg:
+                    ff_rows.append(mat(f + "shared.sg") if L.shared_ff else torch.zeros(1, W, device=device, dtype=dtype))
+                pad = -sum(r.shape[0] for r in ff_rows) % 8
+                if pad:
+                    ff_rows.append(torch.zeros(pad, W, device=device, dtype=dtype))
+                ff_out = [mat(f + n + "down") for n in names]
+                if L.moe_correction:
+                    entry["correction"] = vec(f + "correction")
             else:
                 W = cfg.width
                 shared = [mat(f + "shared.up")] if L.shared_ff else []
