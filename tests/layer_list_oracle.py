@@ -581,7 +581,7 @@ def lovulix_forward(config, W, tokens, streams=None):
                 v_first = v
             else:
                 lam = float(W[m + "vmix"])
-                v = (1.0 - lam) * v + lam * v_first
+                v = ((1.0 - lam) * v.reshape(L, G * V) + lam * v_first.reshape(L, -1)).reshape(L, G, V)  # (token by token, the values of all K/V heads side by side)
         mask = mc.get("mask") or {}
         o = talking_chunk_attention(q, k, v, mc["scale"], W[m + "talk"], W[m + "sink"], mask.get("size")).reshape(L, H * V)
         o = o * sigmoid(x @ W[m + "g"].T)
