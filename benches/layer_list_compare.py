@@ -13,6 +13,11 @@ engine -- at equal width, head count, head width and matrix elements per layer: 
 gated linear attention + mixture of experts, latent attention + gated feed-forward, latent attention on the third layer's cache
 + mixture of experts).  Its roofline counts what the design needs, not what the engine computes: the experts a token takes (not
 all of them), a latent cache row of kv_rank + rot_dim per token.
+
+`--layer-list-family Lovulix` measures the Lovulix family beside Fonapel with attention layers only (the like kernels: the same projections,
+attention over the same paged K/V, one more norm per branch), at equal width, heads, head width and matrix elements a token multiplies:
+4 attention layers (16 heads at width 2048, a quarter of them K/V heads, scores mixed across heads, chunks of 8,192 positions, learned sinks,
+values blended from the second layer on) with 8 gated experts of W / 2 (2 taken) beside a shared one of W.
 """
 
 from __future__ import annotations
@@ -25,13 +30,46 @@ HBM_BYTES_PER_S = 8.0e12
 BF16_FLOPS = 2.5e15
 
 
-def fonapel_config(width: int, layers: int = 4, vocab: int = 32768) -> dict:
+def lovulix_config(width: int, layers: int = 4, vocab: int = 32768, chunk: int = 8192) -> dict:
+    heads = max(1, width // 128)
+    kv = max(1, heads // 4)
+    rot = {"base": 5e5, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    mixer = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "mask": {"size": chunk}, "rot": rot, "scale": 128 ** -0.5, "v_mix": True}
+    mlp = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 8, "top": 2}, "shared": {"ff": width}}
+    return {"architecture": "Lovulix", "layers": [{"type": "attention", "mixer": dict(mixer), "mlp": mlp} for _ in range(layers)], "logit_scale": 1.0,
+            "norm": {"eps": 1e-5}, "vocab": vocab, "width": width}
+
+
+def lovulix_costs(cfg: dict, ctx: int, dtype_bytes: int = 2) -> dict:
+    """What the design needs: the matrix elements a token multiplies (the experts it takes), attention multiply-adds per (query, key) pair of
+    one chunk, the bytes a decode step of b sequences streams (every matrix once, of the experts those b tokens can take; the keys and values of
+    the query's own chunk)."""
+    W, fixed, per_expert, taken, kv_per_tok, attn, chunk = cfg["width"], 0, [], [], 0, 0, 0
+    for L in cfg["layers"]:
+        m, mlp = L["mixer"], L["mlp"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        fixed += W * (H * D + G * D + G * V + H * V) + H * V * W
+        kv_per_tok += G * (D + V)
+        attn += H * (D + V + H)
+        chunk = (m.get("mask") or {}).get("size", 0)
+        if mlp:
+            fixed += W * mlp["router"]["experts"] + (3 * W * mlp["shared"]["ff"] if mlp.get("shared") else 0)
+            per_expert.append(3 * W * mlp["expert"]["ff"])
+            taken.append((mlp["router"]["top"], mlp["router"]["experts"]))
+    head = cfg["vocab"] * W
+    seen = min(ctx, (ctx - 1) % chunk + 1) if chunk else ctx
+    return {"matrix_elems": fixed + sum(pe * top for pe, (top, _) in zip(per_expert, taken)), "head_elems": head, "attn_macs_per_pair": attn, "chunk": chunk,
+            "decode_bytes": lambda b: (fixed + head + sum(pe * min(n, b * top) for pe, (top, n) in zip(per_expert, taken))) * dtype_bytes
+            + b * seen * kv_per_tok * dtype_bytes}
+
+
+def fonapel_config(width: int, layers: int = 4, vocab: int = 32768, order: str = "mixed") -> dict:
     heads = max(1, width // 128)
     kv = max(1, heads // 4)
     attn = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "rot": {"dims": 64, "base": 1e6}, "scale": 128 ** -0.5},
             "mlp": {"kind": "dense", "ff": 3 * width}}
     delta = {"type": "delta", "mixer": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}, "mlp": {"kind": "dense", "ff": 3 * width}}
-    order = [delta, attn, attn, delta]
+    order = [attn] * 4 if order == "attention" else [delta, attn, attn, delta]
     return {"architecture": "Fonapel", "layers": [order[i % 4] for i in range(layers)], "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": vocab,
             "width": width}
 
@@ -162,8 +200,8 @@ def measure(engine, prompt, decode_steps: int, batches=(1, 4), free_running=None
     return out
 
 
-def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, device: str = "cuda") -> dict:
-    """Zefapel beside Fonapel, both on the layer-list engine."""
+def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, device: str = "cuda", family: str = "Zefapel") -> dict:
+    """Zefapel or Lovulix beside Fonapel (Lovulix: beside its attention layers only), all on the layer-list engine."""
     import torch
 
     from tiny_llm_hip.models import engine_for
@@ -177,7 +215,8 @@ def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed
         page = 128
         pages = 4 * ((prompt_len + 3 * decode_steps) // page + 2)
         row = {"width": W, "prompt_len": prompt_len, "decode_steps": decode_steps}
-        for key, cfg, costs in (("zefapel", zefapel_config(W), zefapel_costs), ("fonapel", fonapel_config(W), fonapel_costs)):
+        new = ("zefapel", zefapel_config(W), zefapel_costs) if family == "Zefapel" else ("lovulix", lovulix_config(W), lovulix_costs)
+        for key, cfg, costs in (new, ("fonapel", fonapel_config(W, order="attention" if family == "Lovulix" else "mixed"), fonapel_costs)):
             model = synthetic_layer_list(cfg, seed=seed, device=device)
             eng = engine_for(model, dtype=torch.bfloat16, page_size=page, num_pages=pages, max_batch=4, max_pages_per_seq=pages // 4, max_prefill_rows=prompt_len)
             try:
@@ -188,10 +227,10 @@ def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed
             row[key] = summarize(got, costs(cfg, ctx), prompt_len)
             torch.cuda.empty_cache()
         for leg in ("prefill", "decode_b1", "decode_b4"):
-            a, b = row["zefapel"][leg]["roofline_fraction"], row["fonapel"][leg]["roofline_fraction"]
+            a, b = row[new[0]][leg]["roofline_fraction"], row["fonapel"][leg]["roofline_fraction"]
             row.setdefault("times_as_far_from_roofline", {})[leg] = round(b / a, 2) if a > 0 else None
         results.append(row)
-    return {"bench": "layer_list_compare", "family": "Zefapel", "beside": "Fonapel", "dtype": "bf16", "data": "synthetic",
+    return {"bench": "layer_list_compare", "family": family, "beside": "Fonapel", "dtype": "bf16", "data": "synthetic",
             "roofline": {"hbm_bytes_per_s": HBM_BYTES_PER_S, "bf16_flops": BF16_FLOPS}, "results": results}
 
 
@@ -241,7 +280,9 @@ def run(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, d
 
 
 def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
-    flops = 2.0 * (costs["matrix_elems"] * prompt_len + costs["head_elems"]) + 2.0 * costs["attn_macs_per_pair"] * prompt_len * (prompt_len + 1) / 2
+    chunk = costs.get("chunk") or prompt_len  # a chunked mask: whole chunks and the prompt's last, partial one
+    pairs = (prompt_len // chunk) * chunk * (chunk + 1) / 2 + (prompt_len % chunk) * (prompt_len % chunk + 1) / 2
+    flops = 2.0 * (costs["matrix_elems"] * prompt_len + costs["head_elems"]) + 2.0 * costs["attn_macs_per_pair"] * pairs
     out = {"prefill": {"tokens_per_s": round(prompt_len / got["prefill_s"], 1), "ms": round(got["prefill_s"] * 1e3, 3), "tflops": round(flops / got["prefill_s"] / 1e12, 1),
                        "roofline_fraction": round(flops / got["prefill_s"] / BF16_FLOPS, 4)}}
     for b in (1, 4):
@@ -253,6 +294,7 @@ def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
 
 
 def main(widths, prompt_len=2048, decode_steps=64, family="Fonapel") -> None:
-    if family not in ("Fonapel", "Zefapel"):
+    if family not in ("Fonapel", "Zefapel", "Lovulix"):
         raise SystemExit(f"--layer-list-family: unknown family {family!r}")
-    print(json.dumps((run if family == "Fonapel" else run_family_pair)(widths, prompt_len, decode_steps)), flush=True)
+    out = run(widths, prompt_len, decode_steps) if family == "Fonapel" else run_family_pair(widths, prompt_len, decode_steps, family=family)
+    print(json.dumps(out), flush=True)
