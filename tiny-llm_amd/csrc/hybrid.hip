@@ -325,12 +325,61 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
 }
 
-// attention whose scores are mixed across heads, whose mask is chunked or whose sinks are learned: every query head of a row in one workgroup
+template <typename D, int DK4, int VT, int NG>
+static int launch_attn_talk_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, const Meta &m, const StepShape &sh,
+                                 const float *gate, int ldg, void *out, int ldo, int HGB) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    const int TQB = 16 / HGB, HP = NG * HGB;
+    const size_t lds = std::max((size_t)HP * HP + 4 * (size_t)(16 * (16 * VT + 4) + 16 * (16 * NG + 4)), (size_t)128 + 4 * 64 * 4 * VT) * sizeof(float);
+    int page_shift = -1;
+    for (int b = 0; b < 30; ++b)
+        if ((1 << b) == c.page_size) page_shift = b;
+    const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0;
+    auto kern = attn_talk_tile_kernel<D, DK4, VT, NG>;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    dim3 grid((sh.max_len + TQB - 1) / TQB, 1, sh.n_seqs * sh.n_splits);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.seq_row0, m.seq_slot, m.row_pos, e->table_dev,
+                       c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.talk_dev, L.sink, L.sink_dev, L.chunk, HGB,
+                       sh.keys_per_split, sh.n_splits, gate, ldg, (S *)out, ldo, e->part_acc, e->part_ml, page_shift, vec_ok);
+    TL_CHECK_LAUNCH("hybrid attention tile (mixed heads)");
+    if (sh.n_splits > 1) {
+        hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
+                           ldg, (S *)out, ldo);
+        TL_CHECK_LAUNCH("hybrid attention merge");
+    }
+    return TL_OK;
+}
+
+// attention whose scores are mixed across heads, whose mask is chunked or whose sinks are learned: every query head of a token in one workgroup.
+// The MFMA tile kernel where its templates reach (head groups of at most 16, at most 4 K/V heads -- 8 with narrow heads --, dim and vdim up to 128);
+// the row kernel (a workgroup per row, a wave per head) beyond, and as the A/B twin (TL_HYBRID_ATTN_ROWS=1)
 template <typename D>
 static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, const Meta &m, const StepShape &sh, const float *gate,
                           int ldg, void *out, int ldo) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
+    const int HG = L.heads / L.kv_heads, G = L.kv_heads, dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
+    int HGB = 1;
+    while (HGB < HG) HGB *= 2;
+    const int NG = G <= 1 ? 1 : (G <= 2 ? 2 : (G <= 4 ? 4 : 8));
+    const bool narrow = dk4 <= 16 && vt_n <= 4, mid = dk4 <= 32 && vt_n <= 8;
+    if (!e->attn_rows_only && HGB <= 16 && NG * HGB <= 64 && ((narrow && G <= 8) || (mid && G <= 4))) {
+#define HY_TALK(DK, VTT)                                                                                                   \
+    switch (NG) {                                                                                                          \
+        case 1: return launch_attn_talk_tile<D, DK, VTT, 1>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);          \
+        case 2: return launch_attn_talk_tile<D, DK, VTT, 2>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);          \
+        default: return launch_attn_talk_tile<D, DK, VTT, 4>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);         \
+    }
+        if (narrow) {
+            if (NG == 8) return launch_attn_talk_tile<D, 16, 4, 8>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);
+            HY_TALK(16, 4)
+        }
+        HY_TALK(32, 8)
+#undef HY_TALK
+    }
+    StepShape one = sh;  // (the row kernel walks a row's whole key range)
+    one.n_splits = 1;
     const int nw = std::min(16, L.heads);
     const size_t lds = ((size_t)L.heads * L.dim + (size_t)L.heads * 64 + (size_t)nw * 64) * sizeof(float);
     TL_REQUIRE(lds <= 160 * 1024, "hybrid attention: heads * dim too large for the head-mixing kernel");

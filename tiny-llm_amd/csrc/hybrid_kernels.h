@@ -812,6 +812,308 @@ __global__ __launch_bounds__(1024) void attn_talk_rows_kernel(const float *qbuf,
     }
 }
 
+// ---- attention, step 2 with scores mixed across heads (tile form): MFMA flash attention in which a workgroup owns EVERY query head of its tokens ----
+// Mixing needs the scores of all heads of a (query, key) pair at once, so a workgroup owns TQB = 16 / HGB tokens with all their heads: NG row blocks of 16
+// rows, block g = the query heads of K/V head g (row = token * HGB + head in group, HGB = the group's heads rounded up to a power of two).  The four waves
+// split the KEYS: of every 64-key tile wave w takes keys 16 w .. 16 w + 15, holds all NG row blocks, and keeps its own running (max, sum, O) per row; the
+// four partial sets are merged through LDS at the end.  Nothing in the key loop is shared between waves, so it runs without workgroup barriers.
+// Per tile and wave:
+//   S^T_g[key, row] = K_g . Q_g^T  for g < NG     A = the wave's 16 key rows of K/V head g straight from their pages (a lane's 8 consecutive bfloat16, or
+//                                                 DK4 consecutive float32: a dot product does not care in which order its terms are paired), B = the block's
+//                                                 query rows (bfloat16 pages: v_mfma_f32_16x16x32_bf16 with float32 sums; float32 pages: v_mfma_f32_16x16x4_f32)
+//   mix: the raw scores go to the wave's LDS region as [key][token][head]; every lane reads the heads of its (key, token) back and forms
+//        s'_h = sum_g talk[h, g] s_g for its head in every block (the matrix lies in LDS, padded with zeros to the padded head count; no mixing = identity)
+//   mask (causal; chunked: keys from the first position of the query's chunk), running maximum and sum per row -- the sink is their start value (sink_h, 1)
+//   O^T_g[vcol, row] += V_g^T . P_g^T           A = the wave's 16 rows of V_g staged in its LDS region as float32 (the next block's rows are loaded ahead),
+//                                                 B = the weights where the mix left them (v_mfma_f32_16x16x4_f32)
+// The key range may be split over gridDim.z (decode steps over long contexts): partial sums + (max, sum) go to part_* and attn_merge_kernel finishes.
+template <typename D, int DK4, int VT, int NG>
+__global__ __launch_bounds__(256) void attn_talk_tile_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
+                                                             const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
+                                                             const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
+                                                             float scale, const float *talk, int sink, const float *sinks, int chunk, int HGB,
+                                                             int keys_per_split, int n_splits, const float *gate, int ldg, typename D::storage *out, int ldo,
+                                                             float *part_acc, float *part_ml, int page_shift, int vec_ok) {
+    using S = typename D::storage;
+    extern __shared__ float smem[];
+    constexpr bool KB16 = sizeof(S) == 2;
+    constexpr int VP = 16 * VT + 4, XW = 16 * NG + 4, NITV = VT / 2;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
+    const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+    const int HG = H / G, TQB = 16 / HGB, HP = NG * HGB;
+    const int r0 = seq_row0[seq], len = seq_row0[seq + 1] - r0, t0 = blockIdx.x * TQB;
+    if (t0 >= len) return;
+    float *Tl = smem;                                            // [HP][HP] mixing matrix over padded heads
+    float *Vw = smem + HP * HP + wave * (16 * VP + 16 * XW);     // [16][VP] this wave's value rows of one K/V head
+    float *Sx = Vw + 16 * VP;                                    // [16][XW] this wave's raw scores: [key][token * HP + block * HGB + head in group]
+    for (int i = tid; i < HP * HP; i += 256) {
+        const int tp = i / HP, sp = i % HP, gt = tp / HGB, ht = tp % HGB, gs = sp / HGB, hs = sp % HGB;
+        const bool ok = gt < G && gs < G && ht < HG && hs < HG;
+        Tl[i] = ok ? (talk ? talk[(size_t)(gt * HG + ht) * H + gs * HG + hs] : (tp == sp ? 1.f : 0.f)) : 0.f;
+    }
+    __syncthreads();
+    const int pos0 = row_pos[r0], slot = seq_slot[seq];
+    const int32_t *bt = block_table + (size_t)slot * max_pages;
+    const int tl = col / HGB, hb = col % HGB;
+    const bool row_ok = t0 + tl < len && hb < HG;
+    const int trow = r0 + t0 + tl, qpos = pos0 + t0 + tl;
+    const int qlo = chunk > 0 ? (qpos / chunk) * chunk : 0;
+    const int q_first = pos0 + t0, q_last = pos0 + min(t0 + TQB, len) - 1;
+    const int k_lo = chunk > 0 ? (q_first / chunk) * chunk : 0;
+    const int k_begin = max(k_lo, split * keys_per_split), k_end = min(q_last + 1, (split + 1) * keys_per_split);
+    const bool owns_sink = sink && split == 0 && wave == 0;
+    float m_run[NG], l_run[NG];
+    f32x4 o[NG][VT];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int head = min(g, G - 1) * HG + min(hb, HG - 1);
+        m_run[g] = owns_sink ? (sinks ? sinks[head] : 0.f) : -INFINITY;
+        l_run[g] = owns_sink ? 1.f : 0.f;
+#pragma unroll
+        for (int v = 0; v < VT; ++v) o[g][v] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (k_begin < k_end) {
+        // bfloat16 pages: the B operands of all blocks stay in registers (8 consecutive k per lane and step)
+        u32x4 qb[KB16 ? NG : 1][KB16 ? DK4 / 8 : 1];
+        if constexpr (KB16) {
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                const float *qrow = qbuf + ((size_t)trow * H + (size_t)min(g, G - 1) * HG + min(hb, HG - 1)) * dim;
+                const bool ok = row_ok && g < G;
+#pragma unroll
+                for (int ks8 = 0; ks8 < DK4 / 8; ++ks8)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int d = 32 * ks8 + 8 * g4 + 2 * e;
+                        qb[g][ks8][e] = BF16::pack2((ok && d < dim) ? qrow[d] : 0.f, (ok && d + 1 < dim) ? qrow[d + 1] : 0.f);
+                    }
+            }
+        }
+        // this lane's value chunks of a block: 16 keys x 2 VT chunks of 8 columns, lane + 64 it
+        S vraw[NITV][8];
+        auto load_v = [&](int g, int kb) __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < NITV; ++it) {
+                const int q = lane + 64 * it, j = kb + 16 * wave + q / (2 * VT), c8 = 8 * (q % (2 * VT));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) vraw[it][e] = (S)0;
+                if (g < G && j < k_end && c8 < vdim) {
+                    const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
+                    const S *src = vpool + (((size_t)bt[pg] * G + g) * page_size + in_pg) * vdim + c8;
+                    if (vec_ok) {
+                        if constexpr (KB16) *reinterpret_cast<u32x4 *>(vraw[it]) = *reinterpret_cast<const u32x4 *>(src);
+                        else {
+                            *reinterpret_cast<u32x4 *>(vraw[it]) = *reinterpret_cast<const u32x4 *>(src);
+                            *reinterpret_cast<u32x4 *>(vraw[it] + 4) = *reinterpret_cast<const u32x4 *>(src + 4);
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (c8 + e < vdim) vraw[it][e] = src[e];
+                    }
+                }
+            }
+        };
+        auto store_v = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < NITV; ++it) {
+                const int q = lane + 64 * it;
+                float *dst = Vw + (q / (2 * VT)) * VP + 8 * (q % (2 * VT));
+                f32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = D::to_float(vraw[it][e]);
+                    hi[e] = D::to_float(vraw[it][4 + e]);
+                }
+                *reinterpret_cast<f32x4 *>(dst) = lo;
+                *reinterpret_cast<f32x4 *>(dst + 4) = hi;
+            }
+        };
+        for (int kb = k_begin; kb < k_end; kb += 64) {
+            // ---- raw scores of every block for this wave's 16 keys ----
+            const int jk = kb + 16 * wave + col;  // the key whose row this lane feeds into the A operand
+            const bool key_ok = jk < k_end;
+            const int pgk = key_ok ? (page_shift >= 0 ? (jk >> page_shift) : (jk / page_size)) : 0, in_pgk = jk - pgk * page_size;
+            const size_t krow0 = key_ok ? ((size_t)bt[pgk] * G * page_size + in_pgk) : 0;
+            f32x4 sc[NG];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                f32x4 a4{0.f, 0.f, 0.f, 0.f};
+                const S *kr = kpool + (krow0 + (size_t)min(g, G - 1) * page_size) * dim;
+                const bool ok = key_ok && g < G;
+                if constexpr (KB16) {
+                    u32x4 ka[DK4 / 8];
+#pragma unroll
+                    for (int ks8 = 0; ks8 < DK4 / 8; ++ks8) {
+                        const int d = 32 * ks8 + 8 * g4;
+                        ka[ks8] = u32x4{0u, 0u, 0u, 0u};
+                        if (ok && d < dim) {
+                            if (vec_ok) ka[ks8] = *reinterpret_cast<const u32x4 *>(kr + d);
+                            else {
+                                uint16_t tmp[8];
+#pragma unroll
+                                for (int e = 0; e < 8; ++e) tmp[e] = d + e < dim ? kr[d + e] : (uint16_t)0;
+                                ka[ks8] = *reinterpret_cast<const u32x4 *>(tmp);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int ks8 = 0; ks8 < DK4 / 8; ++ks8)
+                        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[ks8]), __builtin_bit_cast(bf16x8_t, qb[g][ks8]), a4, 0, 0, 0);
+                } else {
+                    // float32 pages: lane group g4 takes the DK4 consecutive dimensions g4 * DK4 .. of its key row and of its query row
+                    const float *qrow = qbuf + ((size_t)trow * H + (size_t)min(g, G - 1) * HG + min(hb, HG - 1)) * dim;
+                    const bool qok = row_ok && g < G;
+#pragma unroll
+                    for (int kk = 0; kk < DK4; ++kk) {
+                        const int d = g4 * DK4 + kk;
+                        const float kv = (ok && d < dim) ? D::to_float(kr[d]) : 0.f;
+                        const float qv = (qok && d < dim) ? qrow[d] : 0.f;
+                        a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kv, qv, a4, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) a4[r] *= scale;
+                sc[g] = a4;
+            }
+            load_v(0, kb);
+            // ---- mix across heads through the wave's LDS region ----
+#pragma unroll
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) Sx[(4 * g4 + r) * XW + tl * HP + g * HGB + hb] = sc[g][r];
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int g = 0; g < NG; ++g) sc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if ((HP & 3) == 0) {
+                for (int sp = 0; sp < HP; sp += 4) {
+                    f32x4 x[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const f32x4 *>(Sx + (4 * g4 + r) * XW + tl * HP + sp);
+#pragma unroll
+                    for (int g = 0; g < NG; ++g) {
+                        const f32x4 c = *reinterpret_cast<const f32x4 *>(Tl + (size_t)(g * HGB + hb) * HP + sp);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) sc[g][r] += c[0] * x[r][0] + c[1] * x[r][1] + c[2] * x[r][2] + c[3] * x[r][3];
+                    }
+                }
+            } else {
+                for (int sp = 0; sp < HP; ++sp) {
+#pragma unroll
+                    for (int g = 0; g < NG; ++g) {
+                        const float c = Tl[(size_t)(g * HGB + hb) * HP + sp];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) sc[g][r] += c * Sx[(4 * g4 + r) * XW + tl * HP + sp];
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            // ---- mask, running maximum and sum per row and block; then the values of each block ----
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                float m_tile = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = kb + 16 * wave + 4 * g4 + r;
+                    sc[g][r] = (row_ok && g < G && j <= qpos && j >= qlo && j < k_end) ? sc[g][r] : -INFINITY;
+                    m_tile = fmaxf(m_tile, sc[g][r]);
+                }
+                m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+                m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+                const float m_new = fmaxf(m_run[g], m_tile);
+                const float corr = (m_run[g] == -INFINITY) ? 0.f : expf(m_run[g] - m_new);
+                float psum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = (sc[g][r] == -INFINITY) ? 0.f : expf(sc[g][r] - m_new);
+                    sc[g][r] = p;
+                    psum += p;
+                }
+                psum += __shfl_xor(psum, 16, 64);
+                psum += __shfl_xor(psum, 32, 64);
+                l_run[g] = l_run[g] * corr + psum;
+                m_run[g] = m_new;
+#pragma unroll
+                for (int v = 0; v < VT; ++v)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[g][v][r] *= corr;
+                store_v();
+                __builtin_amdgcn_wave_barrier();
+                if (g + 1 < NG) load_v(g + 1, kb);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float *vr = Vw + (4 * g4 + r) * VP + col;
+#pragma unroll
+                    for (int v = 0; v < VT; ++v) o[g][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[g][r], o[g][v], 0, 0, 0);
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+    // four waves, four partial sets of the same rows: block by block through LDS (the key loop's regions are no longer needed); wave g & 3 finishes block g
+    float *xm = smem, *xl = smem + 64, *xo = smem + 128;  // [4][16], [4][16], [4][64][4 VT]
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        __syncthreads();
+        if (g4 == 0) {
+            xm[wave * 16 + col] = m_run[g];
+            xl[wave * 16 + col] = l_run[g];
+        }
+#pragma unroll
+        for (int v = 0; v < VT; ++v) *reinterpret_cast<f32x4 *>(xo + ((size_t)(wave * 64 + lane) * VT + v) * 4) = o[g][v];
+        __syncthreads();
+        if (wave != (g & 3) || g >= G) continue;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, xm[w * 16 + col]);
+        float L = 0.f;
+        f32x4 of[VT];
+#pragma unroll
+        for (int v = 0; v < VT; ++v) of[v] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = xm[w * 16 + col];
+            const float f = (mw == -INFINITY) ? 0.f : expf(mw - M);
+            L += xl[w * 16 + col] * f;
+#pragma unroll
+            for (int v = 0; v < VT; ++v) {
+                const f32x4 ow = *reinterpret_cast<const f32x4 *>(xo + ((size_t)(w * 64 + lane) * VT + v) * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) of[v][r] += ow[r] * f;
+            }
+        }
+        if (!row_ok) continue;
+        const int head = g * HG + hb;
+        if (n_splits == 1) {
+            const float invl = L > 0.f ? 1.f / L : 0.f;
+#pragma unroll
+            for (int v = 0; v < VT; ++v)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int c = 16 * v + 4 * g4 + r;
+                    if (c < vdim) {
+                        float val = of[v][r] * invl;
+                        if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (size_t)head * vdim + c]);
+                        out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
+                    }
+                }
+        } else {
+            const size_t pi = ((size_t)trow * H + head) * n_splits + split;
+#pragma unroll
+            for (int v = 0; v < VT; ++v)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int c = 16 * v + 4 * g4 + r;
+                    if (c < vdim) part_acc[pi * vdim + c] = of[v][r];
+                }
+            if (g4 == 0) {
+                part_ml[2 * pi] = M;
+                part_ml[2 * pi + 1] = L;
+            }
+        }
+    }
+}
+
 // ---- the block whose norm sits on the branch's output: x += mult * y / sqrt(mean y^2 + eps) * (offset + w); h = x as D rows (the next sublayer's input) ----
 template <typename D>
 __global__ void postnorm_add_kernel(float *x, const float *y, const float *w, float offset, float eps, float mult, typename D::storage *h, int width) {
