@@ -325,20 +325,25 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
 }
 
-template <typename D, int DK4, int VT, int NG>
+static size_t attn_talk_lds(int es, int DK4, int VT, int G, int HGB) {
+    const size_t HP = (size_t)G * HGB, QP = es == 2 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4;
+    return std::max(HP * HP + (size_t)G * 16 * QP + 4 * (size_t)(16 * (16 * VT + 4) + 16 * (16 * G + 4)), (size_t)128 + 4 * 64 * 4 * VT + 4 * 16 * (16 * VT + 4)) * sizeof(float);
+}
+
+template <typename D, int DK4, int VT, int NP>
 static int launch_attn_talk_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, const Meta &m, const StepShape &sh,
                                  const float *gate, int ldg, void *out, int ldo, int HGB) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
-    const int TQB = 16 / HGB, HP = NG * HGB;
-    const size_t lds = std::max((size_t)HP * HP + 4 * (size_t)(16 * (16 * VT + 4) + 16 * (16 * NG + 4)), (size_t)128 + 4 * 64 * 4 * VT) * sizeof(float);
+    const int TQB = 16 / HGB;
+    const size_t lds = attn_talk_lds((int)sizeof(S), DK4, VT, L.kv_heads, HGB);
     int page_shift = -1;
     for (int b = 0; b < 30; ++b)
         if ((1 << b) == c.page_size) page_shift = b;
     const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0;
-    auto kern = attn_talk_tile_kernel<D, DK4, VT, NG>;
+    auto kern = attn_talk_tile_kernel<D, DK4, VT, NP>;
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    dim3 grid((sh.max_len + TQB - 1) / TQB, 1, sh.n_seqs * sh.n_splits);
+    dim3 grid((sh.max_len + TQB - 1) / TQB, (L.kv_heads + NP - 1) / NP, sh.n_seqs * sh.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.seq_row0, m.seq_slot, m.row_pos, e->table_dev,
                        c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.talk_dev, L.sink, L.sink_dev, L.chunk, HGB,
                        sh.keys_per_split, sh.n_splits, gate, ldg, (S *)out, ldo, e->part_acc, e->part_ml, page_shift, vec_ok);
@@ -352,7 +357,7 @@ static int launch_attn_talk_tile(tl_hybrid *e, const tl_hybrid_layer &L, const v
 }
 
 // attention whose scores are mixed across heads, whose mask is chunked or whose sinks are learned: every query head of a token in one workgroup.
-// The MFMA tile kernel where its templates reach (head groups of at most 16, at most 4 K/V heads -- 8 with narrow heads --, dim and vdim up to 128);
+// The MFMA tile kernel where its templates reach (head groups of at most 16, at most 64 padded heads, dim and vdim up to 128, its LDS within a CU's);
 // the row kernel (a workgroup per row, a wave per head) beyond, and as the A/B twin (TL_HYBRID_ATTN_ROWS=1)
 template <typename D>
 static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, const Meta &m, const StepShape &sh, const float *gate,
@@ -362,24 +367,23 @@ static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     const int HG = L.heads / L.kv_heads, G = L.kv_heads, dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
     int HGB = 1;
     while (HGB < HG) HGB *= 2;
-    const int NG = G <= 1 ? 1 : (G <= 2 ? 2 : (G <= 4 ? 4 : 8));
     const bool narrow = dk4 <= 16 && vt_n <= 4, mid = dk4 <= 32 && vt_n <= 8;
-    if (!e->attn_rows_only && HGB <= 16 && NG * HGB <= 64 && ((narrow && G <= 8) || (mid && G <= 4))) {
+    if (!e->attn_rows_only && HGB <= 16 && G * HGB <= 64 && (narrow || mid) &&
+        attn_talk_lds((int)sizeof(S), narrow ? 16 : 32, narrow ? 4 : 8, G, HGB) <= 160 * 1024) {
+        // blocks a workgroup weighs and multiplies: one for steps of single tokens (a short chain per workgroup, the K/V heads side by side), up to four for prompts
+        const int np = sh.max_len == 1 ? 1 : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
 #define HY_TALK(DK, VTT)                                                                                                   \
-    switch (NG) {                                                                                                          \
+    switch (np) {                                                                                                          \
         case 1: return launch_attn_talk_tile<D, DK, VTT, 1>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);          \
         case 2: return launch_attn_talk_tile<D, DK, VTT, 2>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);          \
         default: return launch_attn_talk_tile<D, DK, VTT, 4>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);         \
     }
         if (narrow) {
-            if (NG == 8) return launch_attn_talk_tile<D, 16, 4, 8>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);
             HY_TALK(16, 4)
         }
         HY_TALK(32, 8)
 #undef HY_TALK
     }
-    StepShape one = sh;  // (the row kernel walks a row's whole key range)
-    one.n_splits = 1;
     const int nw = std::min(16, L.heads);
     const size_t lds = ((size_t)L.heads * L.dim + (size_t)L.heads * 64 + (size_t)nw * 64) * sizeof(float);
     TL_REQUIRE(lds <= 160 * 1024, "hybrid attention: heads * dim too large for the head-mixing kernel");
@@ -452,7 +456,7 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
     if (L.kind == TL_MIX_ATTENTION) {
         const int G = L.kv_heads;
         if (L.qk_norm || L.rot_half || L.v_mix != TL_VMIX_NONE)  // (options of the row-wise preparation; create checked that it covers the layer)
-            hipLaunchKernelGGL((attn_prep_row_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
+            hipLaunchKernelGGL((attn_prep_row_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
                                c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.rot_half, L.qk_norm, L.q_norm_dev, L.k_norm_dev,
                                c.norm_eps, H, G, L.dim, L.vdim, L.v_mix, L.v_mix_lambda, e->vref, e->qbuf, (S *)run.kpool, (S *)run.vpool);
         else

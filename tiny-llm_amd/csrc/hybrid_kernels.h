@@ -677,7 +677,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, c
 // Rotation of the first rot_dims dimensions of each head by pos * inv_freq[i]: pairs (i, i + rot_dims/2) with rot_half, (2i, 2i+1) without.
 // v_mix 1: the row's values are kept in vref [rows, G*vdim]; 2: v <- (1 - lambda) v + lambda vref before they go to their page.
 template <typename D>
-__global__ __launch_bounds__(256) void attn_prep_row_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
+__global__ __launch_bounds__(1024) void attn_prep_row_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
                                                             const int32_t *block_table, int max_pages, int page_size, const float *inv_freq, int rot_dims,
                                                             int rot_half, int qk_norm, const float *qw, const float *kw, float eps, int H, int G, int dim, int vdim,
                                                             int v_mix, float lambda, float *vref, float *qbuf, typename D::storage *kpool,
@@ -691,35 +691,42 @@ __global__ __launch_bounds__(256) void attn_prep_row_kernel(const float *proj, i
     float inv_q = 1.f, inv_k = 1.f;
     if (qk_norm) {
         float sq = 0.f, sk = 0.f;
-        for (int c = tid; c < nq; c += 256) sq += row[c] * row[c];
-        for (int c = tid; c < nk; c += 256) sk += row[nq + c] * row[nq + c];
+        for (int c = tid; c < nq; c += blockDim.x) sq += row[c] * row[c];
+        for (int c = tid; c < nk; c += blockDim.x) sk += row[nq + c] * row[nq + c];
         sq = block_sum(sq, red);
         sk = block_sum(sk, red);
         inv_q = 1.f / sqrtf(sq / (float)nq + eps);
         inv_k = 1.f / sqrtf(sk / (float)nk + eps);
     }
-    const int half = rot_dims / 2;
-    for (int e = tid; e < nq + nk; e += 256) {
-        const bool is_q = e < nq;
-        const int he = is_q ? e : e - nq, hh = he / dim, c = he % dim;
-        const float *src = row + (is_q ? 0 : nq) + (size_t)hh * dim;
-        const float *w = qk_norm ? (is_q ? qw : kw) + (size_t)hh * dim : nullptr;
+    const int half = rot_dims / 2, units = dim - half;  // per head: `half` rotation pairs, then the dimensions that pass
+    for (int e = tid; e < (H + G) * units; e += blockDim.x) {
+        const int hh = e / units, u = e % units;
+        const bool is_q = hh < H;
+        const float *src = row + (size_t)hh * dim;  // (k heads follow the q heads in the row)
+        const float *w = qk_norm ? (is_q ? qw + (size_t)hh * dim : kw + (size_t)(hh - H) * dim) : nullptr;
         const float inv = is_q ? inv_q : inv_k;
-        float val = src[c] * inv * (w ? w[c] : 1.f);
-        if (c < rot_dims) {
-            int partner, fi;
-            bool first;
-            if (rot_half) first = c < half, partner = first ? c + half : c - half, fi = first ? c : c - half;
-            else first = (c & 1) == 0, partner = first ? c + 1 : c - 1, fi = c >> 1;
-            const float other = src[partner] * inv * (w ? w[partner] : 1.f);
+        int c0, c1 = -1;
+        if (u < half) c0 = rot_half ? u : 2 * u, c1 = rot_half ? u + half : 2 * u + 1;
+        else c0 = u + half;
+        float a = src[c0] * inv * (w ? w[c0] : 1.f), b2 = 0.f;
+        if (c1 >= 0) {
+            b2 = src[c1] * inv * (w ? w[c1] : 1.f);
             float sn, cs;
-            sincosf((float)pos * inv_freq[fi], &sn, &cs);
-            val = first ? val * cs - other * sn : val * cs + other * sn;
+            sincosf((float)pos * inv_freq[u], &sn, &cs);
+            const float na = a * cs - b2 * sn, nb = b2 * cs + a * sn;
+            a = na, b2 = nb;
         }
-        if (is_q) qbuf[(size_t)t * nq + he] = val;
-        else kpool[(((size_t)page * G + hh) * page_size + in_page) * dim + c] = D::from_float(val);
+        if (is_q) {
+            float *dst = qbuf + (size_t)t * nq + (size_t)hh * dim;
+            dst[c0] = a;
+            if (c1 >= 0) dst[c1] = b2;
+        } else {
+            typename D::storage *dst = kpool + (((size_t)page * G + (hh - H)) * page_size + in_page) * dim;
+            dst[c0] = D::from_float(a);
+            if (c1 >= 0) dst[c1] = D::from_float(b2);
+        }
     }
-    for (int e = tid; e < nv; e += 256) {
+    for (int e = tid; e < nv; e += blockDim.x) {
         float v = row[nq + nk + e];
         if (v_mix == 1) vref[(size_t)t * nv + e] = v;
         else if (v_mix == 2) v = (1.f - lambda) * v + lambda * vref[(size_t)t * nv + e];
@@ -812,22 +819,24 @@ __global__ __launch_bounds__(1024) void attn_talk_rows_kernel(const float *qbuf,
     }
 }
 
-// ---- attention, step 2 with scores mixed across heads (tile form): MFMA flash attention in which a workgroup owns EVERY query head of its tokens ----
-// Mixing needs the scores of all heads of a (query, key) pair at once, so a workgroup owns TQB = 16 / HGB tokens with all their heads: NG row blocks of 16
-// rows, block g = the query heads of K/V head g (row = token * HGB + head in group, HGB = the group's heads rounded up to a power of two).  The four waves
-// split the KEYS: of every 64-key tile wave w takes keys 16 w .. 16 w + 15, holds all NG row blocks, and keeps its own running (max, sum, O) per row; the
-// four partial sets are merged through LDS at the end.  Nothing in the key loop is shared between waves, so it runs without workgroup barriers.
-// Per tile and wave:
-//   S^T_g[key, row] = K_g . Q_g^T  for g < NG     A = the wave's 16 key rows of K/V head g straight from their pages (a lane's 8 consecutive bfloat16, or
-//                                                 DK4 consecutive float32: a dot product does not care in which order its terms are paired), B = the block's
-//                                                 query rows (bfloat16 pages: v_mfma_f32_16x16x32_bf16 with float32 sums; float32 pages: v_mfma_f32_16x16x4_f32)
+// ---- attention, step 2 with scores mixed across heads (tile form): MFMA flash attention in which a workgroup sees EVERY query head of its tokens ----
+// Mixing needs the scores of all heads of a (query, key) pair at once, so a workgroup owns TQB = 16 / HGB tokens with all their heads: G row blocks of 16
+// rows, block g = the query heads of K/V head g (row = token * HGB + head in group, HGB = the group's heads rounded up to a power of two).  It forms the raw
+// scores of all G blocks, but weights and values only of the NP blocks blockIdx.y * NP ..: prompts take up to four blocks per workgroup, single-token steps
+// one (the chain of a step is short, the raw scores are cheap to repeat).  The four waves split the KEYS: of every 64-key tile wave w takes keys 16 w ..
+// 16 w + 15 and keeps its own running (max, sum, O) per row; the four partial sets are merged through LDS at the end.  Nothing in the key loop is shared
+// between waves but read-only LDS (queries, mixing matrix), so it runs without workgroup barriers.  Per tile and wave:
+//   S^T_g[key, row] = K_g . Q_g^T  for g < G      A = the wave's 16 key rows of K/V head g straight from their pages (a lane's 8 consecutive bfloat16, or
+//                                                 DK4 consecutive float32: a dot product does not care in which order its terms are paired; the next tile's
+//                                                 rows are loaded ahead of the value products), B = the block's query rows from LDS (bfloat16 pages:
+//                                                 v_mfma_f32_16x16x32_bf16 with float32 sums; float32 pages: v_mfma_f32_16x16x4_f32)
 //   mix: the raw scores go to the wave's LDS region as [key][token][head]; every lane reads the heads of its (key, token) back and forms
-//        s'_h = sum_g talk[h, g] s_g for its head in every block (the matrix lies in LDS, padded with zeros to the padded head count; no mixing = identity)
+//        s'_h = sum_g talk[h, g] s_g for its head in each of its blocks (the matrix lies in LDS over the padded heads; no mixing = identity)
 //   mask (causal; chunked: keys from the first position of the query's chunk), running maximum and sum per row -- the sink is their start value (sink_h, 1)
-//   O^T_g[vcol, row] += V_g^T . P_g^T           A = the wave's 16 rows of V_g staged in its LDS region as float32 (the next block's rows are loaded ahead),
+//   O^T_g[vcol, row] += V_g^T . P_g^T           A = the wave's 16 rows of V_g, loaded at the tile's start and staged in its LDS region as float32,
 //                                                 B = the weights where the mix left them (v_mfma_f32_16x16x4_f32)
 // The key range may be split over gridDim.z (decode steps over long contexts): partial sums + (max, sum) go to part_* and attn_merge_kernel finishes.
-template <typename D, int DK4, int VT, int NG>
+template <typename D, int DK4, int VT, int NP>
 __global__ __launch_bounds__(256) void attn_talk_tile_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
                                                              const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
                                                              const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
@@ -837,22 +846,39 @@ __global__ __launch_bounds__(256) void attn_talk_tile_kernel(const float *qbuf, 
     using S = typename D::storage;
     extern __shared__ float smem[];
     constexpr bool KB16 = sizeof(S) == 2;
-    constexpr int VP = 16 * VT + 4, XW = 16 * NG + 4, NITV = VT / 2;
+    constexpr int VP = 16 * VT + 4, NITV = VT / 2;
+    constexpr int QP = KB16 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4;  // floats per query row in LDS (bfloat16 rows: 4 DK4 + 8 16-bit elements)
+    constexpr int NKA = KB16 ? DK4 / 8 : DK4 / 4;               // 16-byte pieces of a key row a lane holds
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
+    // the exponential of a weight: with bfloat16 pages the hardware's (the values it multiplies carry 8 bits); float32 pages keep the exact one
+    auto exp_t = [](float x) __attribute__((always_inline)) { return KB16 ? __expf(x) : expf(x); };
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
-    const int HG = H / G, TQB = 16 / HGB, HP = NG * HGB;
+    const int HG = H / G, TQB = 16 / HGB, HP = G * HGB, XW = 16 * G + 4, g_own0 = blockIdx.y * NP;
     const int r0 = seq_row0[seq], len = seq_row0[seq + 1] - r0, t0 = blockIdx.x * TQB;
     if (t0 >= len) return;
-    float *Tl = smem;                                            // [HP][HP] mixing matrix over padded heads
-    float *Vw = smem + HP * HP + wave * (16 * VP + 16 * XW);     // [16][VP] this wave's value rows of one K/V head
-    float *Sx = Vw + 16 * VP;                                    // [16][XW] this wave's raw scores: [key][token * HP + block * HGB + head in group]
+    float *Tl = smem;                                                       // [HP][HP] mixing matrix over padded heads
+    float *Qs = smem + HP * HP;                                             // [G][16][QP] query rows of every block
+    float *Vw = Qs + (size_t)G * 16 * QP + wave * (16 * VP + 16 * XW);      // [16][VP] this wave's value rows of one K/V head
+    float *Sx = Vw + 16 * VP;                                               // [16][XW] this wave's raw scores: [key][token * HP + block * HGB + head in group]
+    const int pos0 = row_pos[r0], slot = seq_slot[seq];
     for (int i = tid; i < HP * HP; i += 256) {
         const int tp = i / HP, sp = i % HP, gt = tp / HGB, ht = tp % HGB, gs = sp / HGB, hs = sp % HGB;
-        const bool ok = gt < G && gs < G && ht < HG && hs < HG;
+        const bool ok = ht < HG && hs < HG;
         Tl[i] = ok ? (talk ? talk[(size_t)(gt * HG + ht) * H + gs * HG + hs] : (tp == sp ? 1.f : 0.f)) : 0.f;
     }
+    for (int i = tid; i < G * 16 * (2 * DK4); i += 256) {  // pairs of dimensions; rows beyond the chunk's tokens and heads beyond the group are zero
+        const int d = 2 * (i % (2 * DK4)), rw = (i / (2 * DK4)) % 16, g = i / (2 * DK4 * 16);
+        const int t = rw / HGB, h = rw % HGB;
+        const bool ok = t0 + t < len && h < HG;
+        const float *qrow = qbuf + ((size_t)(r0 + t0 + t) * H + (size_t)g * HG + h) * dim;
+        const float a = (ok && d < dim) ? qrow[d] : 0.f, b2 = (ok && d + 1 < dim) ? qrow[d + 1] : 0.f;
+        if constexpr (KB16) reinterpret_cast<uint32_t *>(Qs)[((size_t)g * 16 + rw) * QP + d / 2] = BF16::pack2(a, b2);
+        else {
+            Qs[((size_t)g * 16 + rw) * QP + d] = a * scale;
+            Qs[((size_t)g * 16 + rw) * QP + d + 1] = b2 * scale;
+        }
+    }
     __syncthreads();
-    const int pos0 = row_pos[r0], slot = seq_slot[seq];
     const int32_t *bt = block_table + (size_t)slot * max_pages;
     const int tl = col / HGB, hb = col % HGB;
     const bool row_ok = t0 + tl < len && hb < HG;
@@ -862,207 +888,212 @@ __global__ __launch_bounds__(256) void attn_talk_tile_kernel(const float *qbuf, 
     const int k_lo = chunk > 0 ? (q_first / chunk) * chunk : 0;
     const int k_begin = max(k_lo, split * keys_per_split), k_end = min(q_last + 1, (split + 1) * keys_per_split);
     const bool owns_sink = sink && split == 0 && wave == 0;
-    float m_run[NG], l_run[NG];
-    f32x4 o[NG][VT];
+    float m_run[NP], l_run[NP];
+    f32x4 o[NP][VT];
 #pragma unroll
-    for (int g = 0; g < NG; ++g) {
-        const int head = min(g, G - 1) * HG + min(hb, HG - 1);
-        m_run[g] = owns_sink ? (sinks ? sinks[head] : 0.f) : -INFINITY;
-        l_run[g] = owns_sink ? 1.f : 0.f;
+    for (int i = 0; i < NP; ++i) {
+        const int head = min(g_own0 + i, G - 1) * HG + min(hb, HG - 1);
+        m_run[i] = owns_sink ? (sinks ? sinks[head] : 0.f) : -INFINITY;
+        l_run[i] = owns_sink ? 1.f : 0.f;
 #pragma unroll
-        for (int v = 0; v < VT; ++v) o[g][v] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int v = 0; v < VT; ++v) o[i][v] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     if (k_begin < k_end) {
-        // bfloat16 pages: the B operands of all blocks stay in registers (8 consecutive k per lane and step)
-        u32x4 qb[KB16 ? NG : 1][KB16 ? DK4 / 8 : 1];
-        if constexpr (KB16) {
+        // a lane's pieces of the key rows of four K/V heads (key kb + 16 wave + col): bfloat16 pages: dimensions 32 ks8 + 8 g4 .. + 7; float32 pages:
+        // dimensions g4 * DK4 + 4 c .. + 3
+        u32x4 ka[4][NKA];
+        auto load_k = [&](int gc, int kb) __attribute__((always_inline)) {
+            const int jk = kb + 16 * wave + col;
+            const bool key_ok = jk < k_end;
+            const int pgk = key_ok ? (page_shift >= 0 ? (jk >> page_shift) : (jk / page_size)) : 0, in_pgk = jk - pgk * page_size;
+            const size_t krow0 = key_ok ? ((size_t)bt[pgk] * G * page_size + in_pgk) : 0;
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                const float *qrow = qbuf + ((size_t)trow * H + (size_t)min(g, G - 1) * HG + min(hb, HG - 1)) * dim;
-                const bool ok = row_ok && g < G;
+            for (int gi = 0; gi < 4; ++gi) {
+                const int g = gc + gi;
+                const S *kr = kpool + (krow0 + (size_t)min(g, G - 1) * page_size) * dim;
+                const bool ok = key_ok && g < G;
 #pragma unroll
-                for (int ks8 = 0; ks8 < DK4 / 8; ++ks8)
+                for (int c = 0; c < NKA; ++c) {
+                    const int d = KB16 ? 32 * c + 8 * g4 : g4 * DK4 + 4 * c;
+                    constexpr int NE = KB16 ? 8 : 4;
+                    ka[gi][c] = u32x4{0u, 0u, 0u, 0u};
+                    if (ok && d < dim) {
+                        if (vec_ok) ka[gi][c] = *reinterpret_cast<const u32x4 *>(kr + d);
+                        else {
+                            S tmp[NE];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int d = 32 * ks8 + 8 * g4 + 2 * e;
-                        qb[g][ks8][e] = BF16::pack2((ok && d < dim) ? qrow[d] : 0.f, (ok && d + 1 < dim) ? qrow[d + 1] : 0.f);
+                            for (int e = 0; e < NE; ++e) tmp[e] = d + e < dim ? kr[d + e] : (S)0;
+                            ka[gi][c] = *reinterpret_cast<const u32x4 *>(tmp);
+                        }
                     }
+                }
             }
-        }
-        // this lane's value chunks of a block: 16 keys x 2 VT chunks of 8 columns, lane + 64 it
-        S vraw[NITV][8];
-        auto load_v = [&](int g, int kb) __attribute__((always_inline)) {
+        };
+        // this lane's value chunks of its blocks: 16 keys x 2 VT chunks of 8 columns, lane + 64 it
+        S vraw[NP][NITV][8];
+        auto load_v = [&](int i, int kb) __attribute__((always_inline)) {
 #pragma unroll
             for (int it = 0; it < NITV; ++it) {
-                const int q = lane + 64 * it, j = kb + 16 * wave + q / (2 * VT), c8 = 8 * (q % (2 * VT));
+                const int g = g_own0 + i, q = lane + 64 * it, j = kb + 16 * wave + q / (2 * VT), c8 = 8 * (q % (2 * VT));
 #pragma unroll
-                for (int e = 0; e < 8; ++e) vraw[it][e] = (S)0;
+                for (int e = 0; e < 8; ++e) vraw[i][it][e] = (S)0;
                 if (g < G && j < k_end && c8 < vdim) {
                     const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
                     const S *src = vpool + (((size_t)bt[pg] * G + g) * page_size + in_pg) * vdim + c8;
                     if (vec_ok) {
-                        if constexpr (KB16) *reinterpret_cast<u32x4 *>(vraw[it]) = *reinterpret_cast<const u32x4 *>(src);
+                        if constexpr (KB16) *reinterpret_cast<u32x4 *>(vraw[i][it]) = *reinterpret_cast<const u32x4 *>(src);
                         else {
-                            *reinterpret_cast<u32x4 *>(vraw[it]) = *reinterpret_cast<const u32x4 *>(src);
-                            *reinterpret_cast<u32x4 *>(vraw[it] + 4) = *reinterpret_cast<const u32x4 *>(src + 4);
+                            *reinterpret_cast<u32x4 *>(vraw[i][it]) = *reinterpret_cast<const u32x4 *>(src);
+                            *reinterpret_cast<u32x4 *>(vraw[i][it] + 4) = *reinterpret_cast<const u32x4 *>(src + 4);
                         }
                     } else {
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
-                            if (c8 + e < vdim) vraw[it][e] = src[e];
+                            if (c8 + e < vdim) vraw[i][it][e] = src[e];
                     }
                 }
             }
         };
-        auto store_v = [&]() __attribute__((always_inline)) {
+        load_k(0, k_begin);
 #pragma unroll
-            for (int it = 0; it < NITV; ++it) {
-                const int q = lane + 64 * it;
-                float *dst = Vw + (q / (2 * VT)) * VP + 8 * (q % (2 * VT));
-                f32x4 lo, hi;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    lo[e] = D::to_float(vraw[it][e]);
-                    hi[e] = D::to_float(vraw[it][4 + e]);
-                }
-                *reinterpret_cast<f32x4 *>(dst) = lo;
-                *reinterpret_cast<f32x4 *>(dst + 4) = hi;
-            }
-        };
+        for (int i = 0; i < NP; ++i) load_v(i, k_begin);
         for (int kb = k_begin; kb < k_end; kb += 64) {
-            // ---- raw scores of every block for this wave's 16 keys ----
-            const int jk = kb + 16 * wave + col;  // the key whose row this lane feeds into the A operand
-            const bool key_ok = jk < k_end;
-            const int pgk = key_ok ? (page_shift >= 0 ? (jk >> page_shift) : (jk / page_size)) : 0, in_pgk = jk - pgk * page_size;
-            const size_t krow0 = key_ok ? ((size_t)bt[pgk] * G * page_size + in_pgk) : 0;
-            f32x4 sc[NG];
+            // ---- raw scores of every block for this wave's 16 keys, four K/V heads at a time ----
+            for (int gc = 0; gc < G; gc += 4) {
+                if (gc > 0) load_k(gc, kb);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                f32x4 a4{0.f, 0.f, 0.f, 0.f};
-                const S *kr = kpool + (krow0 + (size_t)min(g, G - 1) * page_size) * dim;
-                const bool ok = key_ok && g < G;
-                if constexpr (KB16) {
-                    u32x4 ka[DK4 / 8];
+                for (int gi = 0; gi < 4; ++gi) {
+                    const int g = gc + gi;
+                    if (g < G) {
+                        f32x4 a4{0.f, 0.f, 0.f, 0.f};
+                        if constexpr (KB16) {
+                            const uint16_t *qr = reinterpret_cast<const uint16_t *>(Qs) + ((size_t)g * 16 + col) * (2 * QP) + 8 * g4;
 #pragma unroll
-                    for (int ks8 = 0; ks8 < DK4 / 8; ++ks8) {
-                        const int d = 32 * ks8 + 8 * g4;
-                        ka[ks8] = u32x4{0u, 0u, 0u, 0u};
-                        if (ok && d < dim) {
-                            if (vec_ok) ka[ks8] = *reinterpret_cast<const u32x4 *>(kr + d);
-                            else {
-                                uint16_t tmp[8];
+                            for (int ks8 = 0; ks8 < DK4 / 8; ++ks8) {
+                                const u32x4 qv = *reinterpret_cast<const u32x4 *>(qr + 32 * ks8);
+                                a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[gi][ks8]), __builtin_bit_cast(bf16x8_t, qv), a4, 0, 0, 0);
+                            }
 #pragma unroll
-                                for (int e = 0; e < 8; ++e) tmp[e] = d + e < dim ? kr[d + e] : (uint16_t)0;
-                                ka[ks8] = *reinterpret_cast<const u32x4 *>(tmp);
+                            for (int r = 0; r < 4; ++r) a4[r] *= scale;
+                        } else {
+                            const float *qr = Qs + ((size_t)g * 16 + col) * QP + g4 * DK4;
+#pragma unroll
+                            for (int c = 0; c < DK4 / 4; ++c) {
+                                const f32x4 qv = *reinterpret_cast<const f32x4 *>(qr + 4 * c);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(ka[gi][c][e]), qv[e], a4, 0, 0, 0);
                             }
                         }
-                    }
 #pragma unroll
-                    for (int ks8 = 0; ks8 < DK4 / 8; ++ks8)
-                        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[ks8]), __builtin_bit_cast(bf16x8_t, qb[g][ks8]), a4, 0, 0, 0);
-                } else {
-                    // float32 pages: lane group g4 takes the DK4 consecutive dimensions g4 * DK4 .. of its key row and of its query row
-                    const float *qrow = qbuf + ((size_t)trow * H + (size_t)min(g, G - 1) * HG + min(hb, HG - 1)) * dim;
-                    const bool qok = row_ok && g < G;
-#pragma unroll
-                    for (int kk = 0; kk < DK4; ++kk) {
-                        const int d = g4 * DK4 + kk;
-                        const float kv = (ok && d < dim) ? D::to_float(kr[d]) : 0.f;
-                        const float qv = (qok && d < dim) ? qrow[d] : 0.f;
-                        a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kv, qv, a4, 0, 0, 0);
+                        for (int r = 0; r < 4; ++r) Sx[(4 * g4 + r) * XW + tl * HP + g * HGB + hb] = a4[r];
                     }
                 }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) a4[r] *= scale;
-                sc[g] = a4;
             }
-            load_v(0, kb);
-            // ---- mix across heads through the wave's LDS region ----
-#pragma unroll
-            for (int g = 0; g < NG; ++g)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) Sx[(4 * g4 + r) * XW + tl * HP + g * HGB + hb] = sc[g][r];
+            if (kb + 64 < k_end) load_k(0, kb + 64);  // lands while the values are multiplied
             __builtin_amdgcn_wave_barrier();
+            // ---- mix across heads for the blocks of this workgroup ----
+            f32x4 sc[NP];
 #pragma unroll
-            for (int g = 0; g < NG; ++g) sc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < NP; ++i) sc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
             if ((HP & 3) == 0) {
                 for (int sp = 0; sp < HP; sp += 4) {
                     f32x4 x[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const f32x4 *>(Sx + (4 * g4 + r) * XW + tl * HP + sp);
 #pragma unroll
-                    for (int g = 0; g < NG; ++g) {
-                        const f32x4 c = *reinterpret_cast<const f32x4 *>(Tl + (size_t)(g * HGB + hb) * HP + sp);
+                    for (int i = 0; i < NP; ++i) {
+                        const f32x4 c = *reinterpret_cast<const f32x4 *>(Tl + (size_t)(min(g_own0 + i, G - 1) * HGB + hb) * HP + sp);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) sc[g][r] += c[0] * x[r][0] + c[1] * x[r][1] + c[2] * x[r][2] + c[3] * x[r][3];
+                        for (int r = 0; r < 4; ++r) sc[i][r] += c[0] * x[r][0] + c[1] * x[r][1] + c[2] * x[r][2] + c[3] * x[r][3];
                     }
                 }
             } else {
                 for (int sp = 0; sp < HP; ++sp) {
 #pragma unroll
-                    for (int g = 0; g < NG; ++g) {
-                        const float c = Tl[(size_t)(g * HGB + hb) * HP + sp];
+                    for (int i = 0; i < NP; ++i) {
+                        const float c = Tl[(size_t)(min(g_own0 + i, G - 1) * HGB + hb) * HP + sp];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) sc[g][r] += c * Sx[(4 * g4 + r) * XW + tl * HP + sp];
+                        for (int r = 0; r < 4; ++r) sc[i][r] += c * Sx[(4 * g4 + r) * XW + tl * HP + sp];
                     }
                 }
             }
             __builtin_amdgcn_wave_barrier();
-            // ---- mask, running maximum and sum per row and block; then the values of each block ----
+            // ---- mask, running maximum and sum per row and block (all blocks first: their lane exchanges overlap) ----
+            float corr[NP];
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
+            for (int i = 0; i < NP; ++i) {
+                const bool blk_ok = row_ok && g_own0 + i < G;
                 float m_tile = -INFINITY;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * wave + 4 * g4 + r;
-                    sc[g][r] = (row_ok && g < G && j <= qpos && j >= qlo && j < k_end) ? sc[g][r] : -INFINITY;
-                    m_tile = fmaxf(m_tile, sc[g][r]);
+                    sc[i][r] = (blk_ok && j <= qpos && j >= qlo && j < k_end) ? sc[i][r] : -INFINITY;
+                    m_tile = fmaxf(m_tile, sc[i][r]);
                 }
                 m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
                 m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-                const float m_new = fmaxf(m_run[g], m_tile);
-                const float corr = (m_run[g] == -INFINITY) ? 0.f : expf(m_run[g] - m_new);
+                const float m_new = fmaxf(m_run[i], m_tile);
+                corr[i] = (m_run[i] == -INFINITY) ? 0.f : (m_new == m_run[i] ? 1.f : exp_t(m_run[i] - m_new));
                 float psum = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float p = (sc[g][r] == -INFINITY) ? 0.f : expf(sc[g][r] - m_new);
-                    sc[g][r] = p;
+                    const float p = (sc[i][r] == -INFINITY) ? 0.f : exp_t(sc[i][r] - m_new);
+                    sc[i][r] = p;
                     psum += p;
                 }
                 psum += __shfl_xor(psum, 16, 64);
                 psum += __shfl_xor(psum, 32, 64);
-                l_run[g] = l_run[g] * corr + psum;
-                m_run[g] = m_new;
+                l_run[i] = l_run[i] * corr[i] + psum;
+                m_run[i] = m_new;
+            }
+            // ---- the values of each block; the block's rows of the next tile are loaded as soon as this tile's are in LDS ----
 #pragma unroll
-                for (int v = 0; v < VT; ++v)
+            for (int i = 0; i < NP; ++i) {
+                if (__any(corr[i] != 1.f && l_run[i] != 0.f)) {  // (most tiles move no row's maximum: the sums keep their scale)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[g][v][r] *= corr;
-                store_v();
+                    for (int v = 0; v < VT; ++v)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[i][v][r] *= corr[i];
+                }
+#pragma unroll
+                for (int it = 0; it < NITV; ++it) {
+                    const int q = lane + 64 * it;
+                    float *dst = Vw + (q / (2 * VT)) * VP + 8 * (q % (2 * VT));
+                    f32x4 lo, hi;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        lo[e] = D::to_float(vraw[i][it][e]);
+                        hi[e] = D::to_float(vraw[i][it][4 + e]);
+                    }
+                    *reinterpret_cast<f32x4 *>(dst) = lo;
+                    *reinterpret_cast<f32x4 *>(dst + 4) = hi;
+                }
                 __builtin_amdgcn_wave_barrier();
-                if (g + 1 < NG) load_v(g + 1, kb);
+                if (kb + 64 < k_end) load_v(i, kb + 64);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const float *vr = Vw + (4 * g4 + r) * VP + col;
 #pragma unroll
-                    for (int v = 0; v < VT; ++v) o[g][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[g][r], o[g][v], 0, 0, 0);
+                    for (int v = 0; v < VT; ++v) o[i][v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[i][r], o[i][v], 0, 0, 0);
                 }
                 __builtin_amdgcn_wave_barrier();
             }
         }
     }
-    // four waves, four partial sets of the same rows: block by block through LDS (the key loop's regions are no longer needed); wave g & 3 finishes block g
+    // four waves, four partial sets of the same rows: block by block through LDS (the key loop's regions are no longer needed); wave i & 3 finishes block i
     float *xm = smem, *xl = smem + 64, *xo = smem + 128;  // [4][16], [4][16], [4][64][4 VT]
 #pragma unroll
-    for (int g = 0; g < NG; ++g) {
+    for (int i = 0; i < NP; ++i) {
         __syncthreads();
         if (g4 == 0) {
-            xm[wave * 16 + col] = m_run[g];
-            xl[wave * 16 + col] = l_run[g];
+            xm[wave * 16 + col] = m_run[i];
+            xl[wave * 16 + col] = l_run[i];
         }
 #pragma unroll
-        for (int v = 0; v < VT; ++v) *reinterpret_cast<f32x4 *>(xo + ((size_t)(wave * 64 + lane) * VT + v) * 4) = o[g][v];
+        for (int v = 0; v < VT; ++v) *reinterpret_cast<f32x4 *>(xo + ((size_t)(wave * 64 + lane) * VT + v) * 4) = o[i][v];
         __syncthreads();
-        if (wave != (g & 3) || g >= G) continue;
+        const int g = g_own0 + i;
+        if (wave != (i & 3) || g >= G) continue;
         float M = -INFINITY;
 #pragma unroll
         for (int w = 0; w < 4; ++w) M = fmaxf(M, xm[w * 16 + col]);
@@ -1082,22 +1113,58 @@ __global__ __launch_bounds__(256) void attn_talk_tile_kernel(const float *qbuf, 
                 for (int r = 0; r < 4; ++r) of[v][r] += ow[r] * f;
             }
         }
-        if (!row_ok) continue;
-        const int head = g * HG + hb;
         if (n_splits == 1) {
+            // the block's 16 rows x vdim through the wave's LDS region, so that a lane writes 8 consecutive columns of one row (and reads its gate as such)
+            float *xt = smem + 128 + 4 * 64 * 4 * VT + (i & 3) * 16 * VP;  // [16][VP], behind the partial sets
             const float invl = L > 0.f ? 1.f / L : 0.f;
 #pragma unroll
-            for (int v = 0; v < VT; ++v)
+            for (int v = 0; v < VT; ++v) {
+                f32x4 t4;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int c = 16 * v + 4 * g4 + r;
-                    if (c < vdim) {
-                        float val = of[v][r] * invl;
-                        if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (size_t)head * vdim + c]);
-                        out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
+                for (int r = 0; r < 4; ++r) t4[r] = of[v][r] * invl;
+                *reinterpret_cast<f32x4 *>(xt + col * VP + 16 * v + 4 * g4) = t4;
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int orow = lane >> 2, otl = orow / HGB, ohb = orow % HGB;
+            if (t0 + otl < len && ohb < HG) {
+                const size_t orow_g = (size_t)(r0 + t0 + otl), ohead = (size_t)g * HG + ohb;
+#pragma unroll
+                for (int k = 0; k < VT / 2; ++k) {
+                    const int c8 = 8 * ((lane & 3) + 4 * k);
+                    if (c8 >= vdim) continue;
+                    const f32x4 lo = *reinterpret_cast<const f32x4 *>(xt + orow * VP + c8), hi = *reinterpret_cast<const f32x4 *>(xt + orow * VP + c8 + 4);
+                    float val[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    const float *gp = gate ? gate + orow_g * ldg + ohead * vdim + c8 : nullptr;
+                    S *op = out + orow_g * ldo + ohead * vdim + c8;
+                    if (vec_ok && (ldg & 3) == 0 && (ldo & 7) == 0 && ((uintptr_t)gate & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+                        if (gp) {
+                            const f32x4 ga = *reinterpret_cast<const f32x4 *>(gp), gb = *reinterpret_cast<const f32x4 *>(gp + 4);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                val[e] *= sigmoid_f(ga[e]);
+                                val[4 + e] *= sigmoid_f(gb[e]);
+                            }
+                        }
+                        S pk[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) pk[e] = D::from_float(val[e]);
+                        if constexpr (KB16) *reinterpret_cast<u32x4 *>(op) = *reinterpret_cast<const u32x4 *>(pk);
+                        else {
+                            *reinterpret_cast<u32x4 *>(op) = *reinterpret_cast<const u32x4 *>(pk);
+                            *reinterpret_cast<u32x4 *>(op + 4) = *reinterpret_cast<const u32x4 *>(pk + 4);
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (c8 + e < vdim) op[e] = D::from_float(gp ? val[e] * sigmoid_f(gp[e]) : val[e]);
                     }
                 }
-        } else {
+            }
+            continue;
+        }
+        if (!row_ok) continue;
+        const int head = g * HG + hb;
+        {
             const size_t pi = ((size_t)trow * H + head) * n_splits + split;
 #pragma unroll
             for (int v = 0; v < VT; ++v)
