@@ -75,6 +75,7 @@ struct tl_hybrid {
     float *part_acc = nullptr, *part_ml = nullptr;  // attention partials of split key ranges: [max_slots, heads, 64, vdim] / [..., 2]
     bool attn_rows_only = false;                    // TL_HYBRID_ATTN_ROWS=1: the one-wave-per-row attention everywhere (A/B twin of the tile kernel)
     float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *obuf = nullptr, *logits = nullptr;
+    unsigned long long *moe_mask = nullptr;  // which experts the rows of a small step take (SegSkip)
     float *y = nullptr;     // [R, width] a branch's result ahead of its norm (the block with the norm on the branch's output)
     float *vref = nullptr;  // [R, G * vdim] the values of the step's rows in the first value-mixing layer
     void *h = nullptr, *cat = nullptr, *cat2 = nullptr, *hsel = nullptr;
@@ -158,7 +159,7 @@ struct NormTail {
 // out (+)= A . W^T by shape: a few rows stream the weights once per column (row kernel), more go through the MFMA tile kernel
 template <typename D>
 static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, int M, int N, int K, int epi, float alpha, const float *bias,
-                    int force, hipStream_t st, int batch = 1, long sa = 0, long sw = 0, long sc = 0, NormTail *tail = nullptr) {
+                    int force, hipStream_t st, int batch = 1, long sa = 0, long sw = 0, long sc = 0, NormTail *tail = nullptr, const SegSkip *skip = nullptr) {
     using S = typename D::storage;
     if (M <= 0 || N <= 0 || batch <= 0) return TL_OK;
     const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && sa % 8 == 0 && sw % 8 == 0;
@@ -189,13 +190,16 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
     S *nout = with_tail ? (S *)tail->out : nullptr;
 #define HY_GEMM(KERN, E) \
     hipLaunchKernelGGL((KERN<D, E>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok, sa, sw, sc, nw, nb, nalpha, nout)
+#define HY_GEMM_ROWS(E) \
+    hipLaunchKernelGGL((gemm_rows_kernel<D, E>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok, sa, sw, sc, nw, nb, nalpha, nout, sk)
     if (rows) {
         dim3 grid((N + 3) / 4, batch), block(256);
-        if (epi == 0) HY_GEMM(gemm_rows_kernel, 0);
-        else if (epi == 1) HY_GEMM(gemm_rows_kernel, 1);
-        else if (epi == 2) HY_GEMM(gemm_rows_kernel, 2);
-        else if (!with_tail) HY_GEMM(gemm_rows_kernel, 3);
-        else HY_GEMM(gemm_rows_kernel, 4);
+        const SegSkip sk = skip ? *skip : SegSkip{};
+        if (epi == 0) HY_GEMM_ROWS(0);
+        else if (epi == 1) HY_GEMM_ROWS(1);
+        else if (epi == 2) HY_GEMM_ROWS(2);
+        else if (!with_tail) HY_GEMM_ROWS(3);
+        else HY_GEMM_ROWS(4);
     } else {
         dim3 grid(((M + 63) / 64) * ((N + 63) / 64), batch), block(256);
         if (epi == 0) HY_GEMM(gemm_tile_kernel, 0);
@@ -205,6 +209,7 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
         else HY_GEMM(gemm_tile_kernel, 4);
     }
 #undef HY_GEMM
+#undef HY_GEMM_ROWS
     if (with_tail) tail->done = true;
     TL_CHECK_LAUNCH("hybrid linear");
     return TL_OK;
@@ -611,9 +616,25 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             TL_CHECK_LAUNCH("hybrid norm on the mixer's output");
             if (L.ff > 0) {
                 const int nin2 = ff_in_cols(L);
-                HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
-                HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
-                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->y, W, rows, W, L.ff, 0, 1.f, nullptr, 0, st));
+                // a step of a few rows takes few experts: the router's rows first, then only the experts some row takes are streamed
+                const bool few = rows <= 8 && L.ff_kind == TL_FF_MOE && L.moe_gated && L.experts <= 64 && L.top < L.experts && L.expert_ff % 8 == 0 && L.shared_ff % 8 == 0 && e->moe_mask;
+                if (few) {
+                    HY_TRY(linear_t<D>(e->h, W, (const S *)L.w_in2_dev + (size_t)2 * L.ff * W, e->proj + 2 * L.ff, nin2, rows, nin2 - 2 * L.ff, W, 0, 1.f, nullptr, 0, st));
+                    hipLaunchKernelGGL(moe_taken_mask_kernel, dim3(1), dim3(256), 0, st, e->proj, nin2, 2 * L.ff, rows, L.experts, L.identity, L.top, L.groups, L.keep,
+                                       L.correction_dev, L.moe_router, e->moe_mask);
+                    TL_CHECK_LAUNCH("hybrid moe taken experts");
+                    SegSkip in_skip, out_skip;
+                    in_skip.mask = out_skip.mask = e->moe_mask;
+                    in_skip.lead = out_skip.lead = L.shared_ff, in_skip.len = out_skip.len = L.expert_ff;
+                    in_skip.period = L.ff, in_skip.limit = 2 * L.ff, out_skip.on_k = 1;
+                    HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, 2 * L.ff, W, 0, 1.f, nullptr, 0, st, 1, 0, 0, 0, nullptr, &in_skip));
+                    HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
+                    HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->y, W, rows, W, L.ff, 0, 1.f, nullptr, 0, st, 1, 0, 0, 0, nullptr, &out_skip));
+                } else {
+                    HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
+                    HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
+                    HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->y, W, rows, W, L.ff, 0, 1.f, nullptr, 0, st));
+                }
                 if (L.ff_kind == TL_FF_MOE && L.identity > 0) {  // identity experts return their input: weight * h joins the branch ahead of its norm
                     hipLaunchKernelGGL((identity_axpy_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->y, (const S *)e->h, e->idw,
                                        (const float *)nullptr, 1.f, W, rows);
@@ -934,7 +955,10 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     e->ld_cat = (max_cat + 7) / 8 * 8;
     HY_TRY(dev_alloc(p, &e->x, (size_t)R * W));
     HY_TRY(dev_alloc(p, &e->x0, (size_t)R * W));
-    if (c.parallel_block == TL_BLOCK_POSTNORM) HY_TRY(dev_alloc(p, &e->y, (size_t)R * W));
+    if (c.parallel_block == TL_BLOCK_POSTNORM) {
+        HY_TRY(dev_alloc(p, &e->y, (size_t)R * W));
+        HY_TRY(dev_alloc(p, &e->moe_mask, 1, true));
+    }
     if (vmix_width > 0) HY_TRY(dev_alloc(p, &e->vref, (size_t)R * vmix_width));
     HY_TRY(dev_alloc(p, &e->proj, (size_t)R * e->ld_proj));
     HY_TRY(dev_alloc(p, &e->qbuf, (size_t)R * std::max(1, max_q)));

@@ -189,23 +189,40 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storag
             }
 }
 
+// Segments of a matrix that a step does not need (the experts no row of a small step takes): bit e of *mask says whether segment e is needed.
+// on_k 0: OUTPUT columns n < limit belong to segment (n % period - lead) / len when n % period >= lead; columns of unneeded segments are not computed
+// (their consumers do not read them).  on_k 1: the K range [lead + e len, lead + (e + 1) len) belongs to segment e; the activations there are zero, so
+// the weights are not read (lead and len are multiples of 8: a 16-byte piece lies in one segment).  At most 64 segments.
+struct SegSkip {
+    const unsigned long long *mask = nullptr;
+    int lead = 0, len = 1, period = 1, limit = 0, on_k = 0;
+};
+
 // ---- row matrix product for a few rows (decode): each wave owns one output column and streams its weight row once ----
 // M <= 8.  Lanes stride over K, 8 elements at a time where the layout allows 16-byte loads.
 template <typename D, int EPI>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
                                                         int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok, long sa, long sw,
-                                                        long sc, const float *nw, const float *nb, float nalpha, typename D::storage *nout) {
+                                                        long sc, const float *nw, const float *nb, float nalpha, typename D::storage *nout,
+                                                        SegSkip skip) {
     using S = typename D::storage;
     A += (size_t)blockIdx.y * sa, W += (size_t)blockIdx.y * sw, out += (size_t)blockIdx.y * sc;
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N) return;
+    const unsigned long long need = skip.mask ? *skip.mask : ~0ull;
+    if (skip.mask && !skip.on_k && n < skip.limit) {
+        const int c = n % skip.period;
+        if (c >= skip.lead && !((need >> ((c - skip.lead) / skip.len)) & 1ull)) return;
+    }
+    const bool k_skip = skip.mask && skip.on_k;
     float acc[8];
 #pragma unroll
     for (int m = 0; m < 8; ++m) acc[m] = 0.f;
     const S *wrow = W + (size_t)n * K;
     if (vec_ok) {
         for (int k = lane * 8; k + 8 <= K; k += 64 * 8) {
+            if (k_skip && k >= skip.lead && !((need >> ((k - skip.lead) / skip.len)) & 1ull)) continue;
             float wf[8];
             if constexpr (sizeof(S) == 2) {
                 u32x4 u = *reinterpret_cast<const u32x4 *>(wrow + k);
@@ -1813,6 +1830,22 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
         const float w = c < ffs ? sgate : sw[(c - ffs) / ffe], u = fmaxf(row[su0 + c], 0.f);
         o[c] = D::from_float(w * u * u);
     }
+}
+// which experts the rows of a small step take: bit e of *mask is set when some row's router takes expert e (the products around the activation then leave the
+// others out, see SegSkip).  One workgroup; experts <= 64.
+__global__ __launch_bounds__(256) void moe_taken_mask_kernel(const float *proj, int ldp, int r0, int rows, int experts, int identity, int top, int groups, int keep,
+                                                             const float *correction, int router, unsigned long long *mask) {
+    __shared__ float sw[256], sc[256];
+    __shared__ float gm[256];
+    __shared__ unsigned long long taken;
+    if (threadIdx.x == 0) taken = 0ull;
+    __syncthreads();
+    for (int t = 0; t < rows; ++t) {
+        moe_route_row(proj + (size_t)t * ldp, r0, experts + identity, top, groups, keep, correction, router, sw, sc, gm);
+        if ((int)threadIdx.x < experts && sw[threadIdx.x] != 0.f) atomicOr(&taken, 1ull << threadIdx.x);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *mask = taken;
 }
 // the same with gated experts, W_down (act(W_gate h) * W_up h): proj columns g0 .. = shared gate [ffs] | expert gates [ffe each], u0 .. = shared up | expert ups,
 // router logits at r0, the shared expert's scalar gate at sg0 (sg0 < 0: the shared expert is not scaled).  The router's weight w_e multiplies the
