@@ -59,6 +59,8 @@ LAYERS = {
     "as_many_kv_heads": O.lovulix_layer(heads=3, kv_heads=3, dim=8, vdim=8, rot_dims=8),
     "one_head": O.lovulix_layer(heads=1, kv_heads=1, dim=32, vdim=40, rot_dims=32),
     "more_heads_than_waves": O.lovulix_layer(heads=20, kv_heads=5, dim=8, vdim=8, rot_dims=4),
+    "eight_kv_heads": O.lovulix_layer(heads=16, kv_heads=8, dim=16, vdim=16, rot_dims=8),        # the value blocks of a prompt over two workgroups, of a decode step over four
+    "sixteen_kv_heads_wide": O.lovulix_layer(heads=16, kv_heads=16, dim=72, vdim=72, rot_dims=32),  # the 128-wide tile, four workgroups of four blocks
     "odd_sizes": O.lovulix_layer(heads=6, kv_heads=2, dim=10, vdim=13, rot_dims=6, chunk=11, mlp=O.lovulix_moe(experts=5, top=2, ff=9, shared=11)),
     "wide_heads": O.lovulix_layer(heads=2, kv_heads=1, dim=136, vdim=130, rot_dims=64),
     "every_expert_taken": O.lovulix_layer(mlp=O.lovulix_moe(experts=3, top=3, ff=16, shared=8)),

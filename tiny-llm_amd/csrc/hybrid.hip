@@ -376,7 +376,7 @@ static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     if (!e->attn_rows_only && HGB <= 16 && G * HGB <= 64 && (narrow || mid) &&
         attn_talk_lds((int)sizeof(S), narrow ? 16 : 32, narrow ? 4 : 8, G, HGB) <= 160 * 1024) {
         // blocks a workgroup weighs and multiplies: one for steps of single tokens (a short chain per workgroup, the K/V heads side by side), up to four for prompts
-        const int np = sh.max_len == 1 ? 1 : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+        const int np = sh.max_len == 1 ? (G > 4 ? 2 : 1) : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
 #define HY_TALK(DK, VTT)                                                                                                   \
     switch (np) {                                                                                                          \
         case 1: return launch_attn_talk_tile<D, DK, VTT, 1>(e, L, kpool, vpool, m, sh, gate, ldg, out, ldo, HGB);          \
