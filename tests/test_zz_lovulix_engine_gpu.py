@@ -61,6 +61,7 @@ LAYERS = {
     "more_heads_than_waves": O.lovulix_layer(heads=20, kv_heads=5, dim=8, vdim=8, rot_dims=4),
     "eight_kv_heads": O.lovulix_layer(heads=16, kv_heads=8, dim=16, vdim=16, rot_dims=8),        # the value blocks of a prompt over two workgroups, of a decode step over four
     "sixteen_kv_heads_wide": O.lovulix_layer(heads=16, kv_heads=16, dim=72, vdim=72, rot_dims=32),  # the 128-wide tile, four workgroups of four blocks
+    "head_group_beyond_the_tile_kernel": O.lovulix_layer(heads=24, kv_heads=1, dim=8, vdim=8, rot_dims=4),   # the row kernel, its waves taking the heads in two passes
     "odd_sizes": O.lovulix_layer(heads=6, kv_heads=2, dim=10, vdim=13, rot_dims=6, chunk=11, mlp=O.lovulix_moe(experts=5, top=2, ff=9, shared=11)),
     "wide_heads": O.lovulix_layer(heads=2, kv_heads=1, dim=136, vdim=130, rot_dims=64),
     "every_expert_taken": O.lovulix_layer(mlp=O.lovulix_moe(experts=3, top=3, ff=16, shared=8)),
@@ -80,6 +81,36 @@ def test_each_mechanism_alone(layer, dtype):
         want = O.lovulix_forward(config, W, toks)
         assert close(whole(engine, toks), want, dtype)
         assert close(in_portions(engine, toks, [9, 1, 2]), want, dtype)
+    finally:
+        engine.close()
+
+
+def test_width_and_vocabulary_that_are_no_multiples_of_8():
+    config = O.lovulix_config([O.lovulix_layer(heads=3, kv_heads=1, dim=10, vdim=6, rot_dims=4, chunk=7, mlp=O.lovulix_moe(experts=3, top=2, ff=5, shared=7))], width=50, vocab=77)
+    W = O.make_lovulix_weights(config, seed=40)
+    toks = tokens_for(config, 33, seed=41)
+    want = O.lovulix_forward(config, W, toks)
+    engine = make_engine(config, W)
+    try:
+        assert rel_err(whole(engine, toks), want) < TOL[torch.float32]
+        assert rel_err(in_portions(engine, toks, [4, 1, 1, 9]), want) < TOL[torch.float32]
+    finally:
+        engine.close()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_kernel_twin_of_the_tile_kernel(dtype, monkeypatch):
+    """TL_HYBRID_ATTN_ROWS=1 sends every attention layer through the row kernels (a workgroup per row, a wave per head): the twin of the
+    MFMA tile kernel gives the same logits, in prompts, portions and single tokens."""
+    monkeypatch.setenv("TL_HYBRID_ATTN_ROWS", "1")
+    config = for_dtype(MIXED, dtype)
+    W = O.make_lovulix_weights(config, seed=42)
+    toks = tokens_for(config, 70, seed=43)
+    want = O.lovulix_forward(config, W, toks)
+    engine = make_engine(config, W, dtype)
+    try:
+        assert close(whole(engine, toks), want, dtype)
+        assert close(in_portions(engine, toks, [33, 1, 2, 1]), want, dtype)
     finally:
         engine.close()
 
