@@ -327,13 +327,15 @@ def test_keys_just_inside_and_just_outside_a_chunk(needle_at, seen, query):
     _needle_case(config, W, A, B, 256, needle_at, query, seen, page_size=16, num_pages=24, max_batch=1)
 
 
-@pytest.mark.parametrize("n,needle_at,seen", [(101, 99, False), (150, 99, False), (150, 100, True), (201, 199, False), (199, 100, True), (199, 99, False), (200, 101, True)])
+@pytest.mark.parametrize("n,needle_at,seen", [(101, 99, False), (150, 99, False), (150, 100, True), (201, 199, False), (199, 100, True), (199, 99, False), (200, 101, True),
+                                              (450, 399, False), (450, 400, True), (450, 447, True), (450, 448, True)])
 @pytest.mark.parametrize("query", ["prompt", "decoded"])
 def test_chunk_edges_that_are_no_page_or_tile_edges(n, needle_at, seen, query):
     """Chunks of 100 positions: their edges fall inside pages and inside the kernels' 64-key tiles; a query that is the first of its
-    chunk (position 100, 200) sees only itself."""
+    chunk (position 100, 200) sees only itself.  At 450 tokens a decoded token's key range is split over workgroups (64 keys each): most
+    splits lie before the chunk and hold nothing but -- the first one -- the sink; the chunk starts inside one."""
     config, W, A, B = _needle_model(chunk=100)
-    _needle_case(config, W, A, B, n, needle_at, query, seen, page_size=16, num_pages=24, max_batch=1)
+    _needle_case(config, W, A, B, n, needle_at, query, seen, page_size=16, num_pages=30, max_batch=1)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
