@@ -16,7 +16,11 @@
  *                      (rot_scaling_kind 1), scores mixed across query heads before the softmax (talk_dev), a learned
  *                      sink logit per head (sink_dev), a chunked causal mask (chunk: a query sees the keys of its own
  *                      run of `chunk` positions only), values blended with the values the first such layer computed for
- *                      the same token (v_mix).
+ *                      the same token (v_mix).  Also: biases on the projections (w_in_bias_dev), an RMS norm per head with one [dim] weight
+ *                      before the rotation (qk_head_norm), a sliding window (window: a query sees itself and the window - 1 keys
+ *                      before it), one gate number per head (gated 2), and differential attention (diff_maps): every head has two
+ *                      query / key maps [map 1 | map 2] over the same values, each an attention of its own; the read-outs combine
+ *                      as a1 - lambda a2, are divided by their RMS over vdim and multiplied by 1 - diff_init.
  *   TL_MIX_DELTA       gated delta rule: a [key_dim, value_dim] float32 state per head that decays, is corrected
  *                      towards the new value along the new key and is read with the query; q/k/v pass a short
  *                      causal depthwise convolution + SiLU first.  The state and the convolution's last inputs
@@ -29,6 +33,9 @@
  *                      cap tanh(x / cap), with a running maximum m (starting at 0) that keeps them in range, and a
  *                      normaliser n_t = a n + b k: o / (max(|n.q|, e^-m) + 1e-6) (the matrix memory of xLSTM); the
  *                      read-out is unit-RMS per head, times a [heads*vdim] weight, gated by a sigmoid.
+ *                      rec_kind TL_REC_FIXED: one constant decay per head (decay_dev), b = 1, no normaliser (retention); q and k
+ *                      may carry rotary positions on their first rot_dims dimensions and k (not q) is scaled by dim^-1/2; the
+ *                      read-out is unit-RMS per head without a weight (out_norm_dev NULL) and gated by SiLU.
  *                      State (and m) live in the state slot of the sequence.
  *   TL_MIX_LATENT      latent attention: queries through a normed low-rank latent; keys and values are per-head
  *                      projections (W_uk, W_uv) of ONE normed latent c [kv_rank] per token, plus one rotated key part
@@ -40,15 +47,18 @@
  *
  * Block forms: parallel_block 1 is x += m (mixer(h) + ff(h)) with one norm; 0 is the sequential pre-norm block
  * x += ls1 * mixer(norm1 x); x += ls2 * ff(norm2 x) with optional per-channel scales ls1 / ls2; 2 is the block with the norm on
- * the branch's OUTPUT, x += m norm1(mixer(x)); x += m norm2(ff(x)), whose sublayers read the stream itself.  Norms: RMS or
+ * the branch's OUTPUT, x += m norm1(mixer(x)); x += m norm2(ff(x)), whose sublayers read the stream itself; 3 has a norm on both sides
+ * of every sublayer, x += m ls1 post1(mixer(norm1 x)); x += m ls2 post2(ff(norm2 x)).  A layer may end with a per-layer token input
+ * (side_*): e = the layer's columns of a second embedding table, y = W_proj (gelu_tanh(W_gate x) * e), x += y / rms(y) * side_norm.
+ * The embedding output may pass an RMS norm (embed_norm_dev).  Norms: RMS or
  * Dynamic Tanh (tanh(alpha x) w + b).  Feed-forward kinds: W_down act(W_up h), W_down (act(W_gate h) * W_up h), or a
  * mixture of experts (softmax or sigmoid router with a selection-only correction, groups of neighbouring experts, identity
  * experts, a shared expert with or without a scalar gate; experts W_down act(W_up h) or, with moe_gated, W_down (act(W_gate h) *
  * W_up h); the router's weight on the expert's output or, with moe_scale_input, on its input).
  *
  * A contiguous range of layers may be repeated ("loop"): each pass has its own K/V pages / state slots, and is
- * entered through a [width, 2 width] projection of the running stream beside the embedding output plus a per-pass
- * offset vector.
+ * entered through a [width, 2 width] projection of the running stream beside the embedding output (loop_in_dev; NULL:
+ * the stream passes as it is) plus a per-pass offset vector.
  *
  * One step function serves prefill, decode and any mixture: tl_hybrid_step takes chunks of token ids for several
  * sequence slots (a chunk of one token is a decode step), runs them as one packed batch of rows and returns the
@@ -74,22 +84,23 @@ extern "C" {
 typedef struct tl_hybrid tl_hybrid;
 
 enum { TL_MIX_ATTENTION = 0, TL_MIX_DELTA = 1, TL_MIX_LINREC = 2, TL_MIX_LATENT = 3 };
-enum { TL_REC_CHANNEL = 0, TL_REC_EXPGATE = 1 };
+enum { TL_REC_CHANNEL = 0, TL_REC_EXPGATE = 1, TL_REC_FIXED = 2 };
 enum { TL_NORM_RMS = 0, TL_NORM_DYT = 1 };
 enum { TL_FF_PLAIN = 0, TL_FF_GATED = 1, TL_FF_MOE = 2 };
 enum { TL_ROUTER_SOFTMAX = 0, TL_ROUTER_SIGMOID = 1 };
-enum { TL_BLOCK_SEQUENTIAL = 0, TL_BLOCK_PARALLEL = 1, TL_BLOCK_POSTNORM = 2 };
+enum { TL_BLOCK_SEQUENTIAL = 0, TL_BLOCK_PARALLEL = 1, TL_BLOCK_POSTNORM = 2, TL_BLOCK_SANDWICH = 3 };
 enum { TL_VMIX_NONE = 0, TL_VMIX_FIRST = 1, TL_VMIX_BLEND = 2 };
 enum { TL_ACT_GELU_ERF = 0, TL_ACT_GELU_TANH = 1, TL_ACT_SILU = 2, TL_ACT_RELU2 = 3 };
 enum { TL_HY_F32 = 0, TL_HY_BF16 = 2 }; /* the values of tl_dtype in tinyllm_hip.h */
 
 /* One layer.  Matrices are [out, in] row-major in the engine's dtype; vectors are float32.
  * w_in: every projection that reads the normed input, rows concatenated in this order:
- *   attention: q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | gate (heads*vdim, if gated) | up (ff, if ff > 0)
+ *   attention: q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | gate (heads*vdim if gated 1, heads if gated 2) | up (ff, if ff > 0)
+ *              with diff_maps: q (heads*2*dim, per head [map 1 | map 2]) | k (kv_heads*2*dim, likewise) | v | gate
  *   delta:     q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | gate (heads*vdim) | a (heads) | b (heads) | up (ff)
  *   linrec:    q (heads*dim) | k (heads*dim) | v (heads*vdim) | gate (heads*vdim) | expgate: i (heads) | f (heads)
- *                                                                                    | channel: a1 (a_rank)
- *   latent:    dq (q_rank) | dkv (kv_rank + rot_dim, unless kv_from >= 0) | gate (heads*vdim)
+ *                                                                                    | channel: a1 (a_rank) | fixed: nothing
+ *   latent:    dq (q_rank) | dkv (kv_rank + rot_dim, unless kv_from >= 0) | gate (heads*vdim, if gated)
  * w_out: [width, heads*vdim + ff]: the mixer's output projection beside the feed-forward's down projection, so
  *   one product yields mixer(h) + ff(h).
  * Sequential block (parallel_block 0): w_in / w_out hold the mixer's rows / columns only; the feed-forward reads
@@ -114,7 +125,7 @@ typedef struct tl_hybrid_layer {
     float scale;
     int qk_unit_rms;        /* q and k divided by their RMS over dim after the rotation */
     int sink;               /* softmax denominator += 1 */
-    int gated;              /* output * sigmoid(gate) */
+    int gated;              /* 1: output * sigmoid(gate), a gate per output channel; 2: one gate per head */
     /* delta */
     int conv_taps;
     const float *conv_dev;  /* [2*kv_heads*dim + heads*vdim, taps], last tap = current token */
@@ -165,6 +176,22 @@ typedef struct tl_hybrid_layer {
     int moe_gated;          /* experts (and the shared one) are W_down (act(W_gate h) * W_up h) */
     int moe_scale_input;    /* the router's weight multiplies the expert's input: expert(w h) */
     int moe_shared_sg;      /* the shared expert is scaled by sigmoid of a scalar projection (its row follows the router's) */
+    /* attention, further options (2) */
+    const float *w_in_bias_dev; /* [the mixer's rows of w_in] added in the projection; NULL: none */
+    int window;             /* > 0: query i sees key j <= i only if i - j < window */
+    int qk_head_norm;       /* 1: every head (and map) of q and k passes an RMS norm over dim with the weights q_norm_dev / k_norm_dev [dim],
+                               before the rotation */
+    int diff_maps;          /* 1: differential attention (two maps per head, see above); the row's gate is applied after the combination */
+    float diff_lambda, diff_init;
+    /* linear recurrence with a constant decay per head (rec_kind TL_REC_FIXED; rotation by rot_dims / rot_base / rot_half / rot_factor ...) */
+    const float *decay_dev; /* [heads] */
+    /* the block with norms on both sides of a sublayer (TL_BLOCK_SANDWICH): RMS weights on the mixer's / feed-forward's result */
+    const float *post_norm_dev, *post_norm2_dev; /* [width] */
+    /* per-layer token input (all NULL / 0: none) */
+    const void *side_gate_dev;  /* [side_dim, width] engine dtype */
+    const void *side_proj_dev;  /* [width, side_dim] engine dtype */
+    const float *side_norm_dev; /* [width], plain weight */
+    int side_col0;              /* first of the layer's side_dim columns in the side embedding table */
 } tl_hybrid_layer;
 
 typedef struct tl_hybrid_config {
@@ -186,6 +213,9 @@ typedef struct tl_hybrid_config {
     const float *final_norm_bias_dev;
     int page_size, num_pages, max_slots, max_pages_per_seq, max_rows;
     float logit_scale;          /* logits = head . norm(x) * logit_scale (0 is read as 1) */
+    const float *embed_norm_dev; /* [width]: x = rms_norm(embed[token] * embed_scale) * (final_norm_offset + w); NULL: none */
+    const void *side_embed_dev;  /* [vocab, side_cols] engine dtype: the table of the per-layer token inputs */
+    int side_cols, side_dim;     /* columns of a table row; columns one layer reads */
 } tl_hybrid_config;
 
 typedef struct tl_hybrid_stats {

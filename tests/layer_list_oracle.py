@@ -654,3 +654,138 @@ def lovulix_layer(heads=4, kv_heads=2, dim=16, vdim=24, rot_dims=8, base=5000.0,
 
 def lovulix_config(layers, width=64, vocab=101, eps=1e-5, logit_scale=0.7):
     return {"architecture": "Lovulix", "layers": layers, "logit_scale": logit_scale, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+# ---- Muduvik: x = norm(embed[token]); layers with a norm before AND after each sublayer and per-channel layer scales; a per-layer token
+# ---- input behind the feed-forward; a looped range entered by adding a per-pass vector.  Mixers: differential sliding-window attention,
+# ---- latent attention without positions, retention.  Same conventions: float64, whole sequences, one function per mechanism. ---------
+
+def window_softmax_attention(q, k, v, scale, window=None):
+    """q [L, H, D], k [L, G, D], v [L, G', V] (head h reads key head h // (H/G) and value head h // (H/G')): query i sees keys j with
+    0 <= i - j < window (None: every j <= i); ordinary softmax.  Row by row."""
+    L, H, _ = q.shape
+    G, Gv = k.shape[1], v.shape[1]
+    out = np.zeros((L, H, v.shape[2]))
+    for h in range(H):
+        for i in range(L):
+            lo = max(0, i - window + 1) if window else 0
+            s = (k[lo:i + 1, h // (H // G)] @ q[i, h]) * scale
+            e = np.exp(s - s.max())
+            out[i, h] = (e / e.sum()) @ v[lo:i + 1, h // (H // Gv)]
+    return out
+
+
+def differential_combine(a1, a2, lam, diff, eps):
+    """a1, a2 [L, H, V]: the two maps' read-outs.  o = a1 - lam a2, divided by its root mean square over V (eps inside the root), times (1 - diff)."""
+    o = a1 - lam * a2
+    return o / np.sqrt(np.mean(o * o, axis=-1, keepdims=True) + eps) * (1.0 - diff)
+
+
+def differential_attention(W, m, mc, h, pos, eps):
+    """The whole mixer on its input h [L, width] -> [L, width]: two maps per head over shared values, sliding window, per-head gate."""
+    L = h.shape[0]
+    H, G, D, V = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+    q = (h @ W[m + "q"].T + W[m + "q.b"]).reshape(L, H, 2, D)
+    k = (h @ W[m + "k"].T + W[m + "k.b"]).reshape(L, G, 2, D)
+    v = (h @ W[m + "v"].T + W[m + "v.b"]).reshape(L, G, V)
+    q, k = rms_norm(q, W[m + "q.norm"], eps), rms_norm(k, W[m + "k.norm"], eps)
+    rot = mc.get("rot")
+    if rot and rot.get("dims", 0):
+        f = wavelength_scaled_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
+        q = rotate_pairs_by(q.reshape(L, 2 * H, D), pos, f).reshape(L, H, 2, D)
+        k = rotate_pairs_by(k.reshape(L, 2 * G, D), pos, f).reshape(L, G, 2, D)
+    window = (mc.get("mask") or {}).get("size")
+    a = [window_softmax_attention(q[:, :, j], k[:, :, j], v, mc["scale"], window) for j in (0, 1)]
+    lam = math.exp(float(W[m + "lq1"] @ W[m + "lk1"])) - math.exp(float(W[m + "lq2"] @ W[m + "lk2"])) + mc["diff"]
+    o = differential_combine(a[0], a[1], lam, mc["diff"], eps)
+    o = o * sigmoid(h @ W[m + "g"].T)[:, :, None]
+    return o.reshape(L, H * V) @ W[m + "o"].T
+
+
+def latent_attention_plain(W, m, mc, h, eps):
+    """Queries through a normed latent; keys and values are per-head projections of one normed latent per token; causal softmax; no positions."""
+    L = h.shape[0]
+    H, D, V = mc["heads"], mc["dim"], mc["vdim"]
+    q = (rms_norm(h @ W[m + "dq"].T, W[m + "dq.norm"], eps) @ W[m + "uq"].T).reshape(L, H, D)
+    c = rms_norm(h @ W[m + "dkv"].T, W[m + "dkv.norm"], eps)
+    k, v = (c @ W[m + "uk"].T).reshape(L, H, D), (c @ W[m + "uv"].T).reshape(L, H, V)
+    return causal_softmax_attention(q, k, v, mc["scale"]).reshape(L, H * V) @ W[m + "o"].T
+
+
+def retention_states(q, k, v, decay):
+    """q, k [L, H, D], v [L, H, V], decay [H].  Per head, token by token, from a zero state: S <- decay S + k v^T;  o = S^T q."""
+    L, H, V = v.shape
+    D = q.shape[2]
+    out = np.zeros((L, H, V))
+    for h in range(H):
+        S = np.zeros((D, V))
+        for t in range(L):
+            S = decay[h] * S + np.outer(k[t, h], v[t, h])
+            out[t, h] = S.T @ q[t, h]
+    return out
+
+
+def retention(W, m, mc, h, pos, eps):
+    L = h.shape[0]
+    H, D, V = mc["heads"], mc["dim"], mc["vdim"]
+    q, k, v = (h @ W[m + "q"].T).reshape(L, H, D), (h @ W[m + "k"].T).reshape(L, H, D), (h @ W[m + "v"].T).reshape(L, H, V)
+    rot = mc.get("rot")
+    if rot and rot.get("dims", 0):
+        f = wavelength_scaled_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
+        q, k = rotate_halves_by(q, pos, f), rotate_halves_by(k, pos, f)
+    o = retention_states(q, k * D ** -0.5, v, np.asarray(mc["decay"], dtype=np.float64))
+    o = rms_norm(o, None, eps).reshape(L, H * V) * silu(h @ W[m + "g"].T)
+    return o @ W[m + "o"].T
+
+
+def token_side_input(W, p, x, side_rows, eps):
+    """side_rows [L, dim]: the layer's part of the side embedding of each token.  y = W_proj (gelu_tanh(W_gate x) * e); returns rms_norm(y) * norm."""
+    y = (gelu_tanh(x @ W[p + "side.gate"].T) * side_rows) @ W[p + "side.proj"].T
+    return rms_norm(y, W[p + "side.norm"], eps)
+
+
+def muduvik_layer_order(config):
+    """(layer index, pass or None, first of its pass) for every layer run."""
+    n, lp = len(config["layers"]), config.get("loop")
+    if not lp:
+        return [(i, None, False) for i in range(n)]
+    runs = [(i, None, False) for i in range(lp["start"])]
+    for t in range(lp["times"]):
+        runs += [(i, t, i == lp["start"]) for i in range(lp["start"], lp["stop"])]
+    return runs + [(i, None, False) for i in range(lp["stop"], n)]
+
+
+def muduvik_forward(config, W, tokens, streams=None):
+    """Logits [L, vocab] of a whole sequence; ``streams`` (a list) receives the residual stream after every layer run."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps = config["norm"]["eps"]
+    tokens = np.asarray(tokens)
+    L = len(tokens)
+    pos = np.arange(L, dtype=np.float64)
+    x = rms_norm(W["embed"][tokens], W["embed.norm"], eps)
+    sd = (config.get("token_side") or {}).get("dim", 0)
+    for i, t, first in muduvik_layer_order(config):
+        if first:
+            x = x + W["loop.step"][t]
+        spec = config["layers"][i]
+        p, m, mc = f"l{i}.", f"l{i}.mix.", spec["mixer"]
+        h = rms_norm(x, W[p + "norm1"], eps)
+        if spec["type"] == "attention":
+            y = differential_attention(W, m, mc, h, pos, eps)
+        elif spec["type"] == "latent_attention":
+            y = latent_attention_plain(W, m, mc, h, eps)
+        elif spec["type"] == "retention":
+            y = retention(W, m, mc, h, pos, eps)
+        else:
+            raise ValueError(spec["type"])
+        x = x + rms_norm(y, W[p + "norm1b"], eps) * W[p + "ls1"]
+        if spec.get("mlp"):
+            h = rms_norm(x, W[p + "norm2"], eps)
+            f = p + "mlp."
+            y = (gelu_tanh(h @ W[f + "gate"].T) * (h @ W[f + "up"].T)) @ W[f + "down"].T
+            x = x + rms_norm(y, W[p + "norm2b"], eps) * W[p + "ls2"]
+        if sd:
+            x = x + token_side_input(W, p, x, W["side.embed"][tokens][:, i * sd:(i + 1) * sd], eps)
+        if streams is not None:
+            streams.append(x.copy())
+    return rms_norm(x, W["final.norm"], eps) @ W["head"].T

@@ -101,10 +101,13 @@ namespace hy {
 
 static size_t esize(int dtype) { return dtype == TL_HY_BF16 ? 2 : 4; }
 
+static int attn_maps(const tl_hybrid_layer &L) { return L.diff_maps ? 2 : 1; }  // query / key maps per head
+static int gate_cols(const tl_hybrid_layer &L) { return L.gated == 2 ? L.heads : (L.gated ? L.heads * L.vdim : 0); }
 static int mixer_cols(const tl_hybrid_layer &L) {  // rows of w_in that belong to the mixer
-    if (L.kind == TL_MIX_ATTENTION) return L.heads * L.dim + L.kv_heads * L.dim + L.kv_heads * L.vdim + (L.gated ? L.heads * L.vdim : 0);
-    if (L.kind == TL_MIX_LINREC) return 2 * L.heads * L.dim + 2 * L.heads * L.vdim + (L.rec_kind == TL_REC_EXPGATE ? 2 * L.heads : L.a_rank);
-    if (L.kind == TL_MIX_LATENT) return L.q_rank + (L.kv_from < 0 ? L.kv_rank + L.rot_dim : 0) + L.heads * L.vdim;
+    if (L.kind == TL_MIX_ATTENTION) return attn_maps(L) * (L.heads + L.kv_heads) * L.dim + L.kv_heads * L.vdim + gate_cols(L);
+    if (L.kind == TL_MIX_LINREC)
+        return 2 * L.heads * L.dim + 2 * L.heads * L.vdim + (L.rec_kind == TL_REC_EXPGATE ? 2 * L.heads : (L.rec_kind == TL_REC_CHANNEL ? L.a_rank : 0));
+    if (L.kind == TL_MIX_LATENT) return L.q_rank + (L.kv_from < 0 ? L.kv_rank + L.rot_dim : 0) + (L.gated ? L.heads * L.vdim : 0);
     return 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads;
 }
 static int ff_in_cols(const tl_hybrid_layer &L) {  // rows of the feed-forward's input matrix
@@ -278,9 +281,27 @@ static void plan_splits(StepShape &sh, int ctx_bound) {
     sh.keys_per_split = kps;
 }
 
+// what the attention core needs beyond the layer's sizes (the defaults are plain causal attention into D rows)
+struct AttnExtra {
+    int window = 0;          // > 0: sliding window
+    int vshare = 1;          // K/V heads in a row that read one value head
+    int gate_per_head = 0;   // the gate holds one number per head
+    float *out32 = nullptr;  // float32 read-out [rows, heads, vdim] instead of D rows
+};
+
+// a windowed layer's split of the keys: a decode step sees at most `window` keys, whatever the context
+static StepShape window_shape(const StepShape &sh, int window) {
+    StepShape w = sh;
+    if (window > 0 && sh.n_splits > 1) {
+        const long covered = (long)sh.n_splits * sh.keys_per_split;
+        plan_splits(w, (int)std::min<long>(covered, window));
+    }
+    return w;
+}
+
 template <typename D, int DK4, int VT>
 static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, int v_row, const Meta &m, const StepShape &sh,
-                            const float *gate, int ldg, void *out, int ldo) {
+                            const float *gate, int ldg, void *out, int ldo, const AttnExtra &x) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     const int HG = L.heads / L.kv_heads;
@@ -300,11 +321,11 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *
     dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.seq_row0, m.seq_slot, m.row_pos,
                        e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.sink, HGB, n_hblk, sh.keys_per_split,
-                       sh.n_splits, gate, ldg, (S *)out, ldo, e->part_acc, e->part_ml, page_shift, vec_ok, v_row);
+                       sh.n_splits, gate, ldg, (S *)out, ldo, e->part_acc, e->part_ml, page_shift, vec_ok, v_row, x.window, x.vshare, x.gate_per_head, x.out32);
     TL_CHECK_LAUNCH("hybrid attention tile");
     if (sh.n_splits > 1) {
         hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
-                           ldg, (S *)out, ldo);
+                           ldg, (S *)out, ldo, x.gate_per_head, x.out32);
         TL_CHECK_LAUNCH("hybrid attention merge");
     }
     return TL_OK;
@@ -312,22 +333,23 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *
 
 // the attention core over one K/V pool by head widths: the MFMA tile kernel where its templates reach, the row kernel beyond
 template <typename D>
-static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, int v_row, const Meta &m, const StepShape &sh,
-                          const float *gate, int ldg, void *out, int ldo) {
+static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, int v_row, const Meta &m, const StepShape &sh0,
+                          const float *gate, int ldg, void *out, int ldo, const AttnExtra &x = AttnExtra{}) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
+    const StepShape sh = window_shape(sh0, x.window);
     const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
     if (e->attn_rows_only || dk4 > 64 || vt_n > 16) {
         hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(sh.rows, L.heads), dim3(64), (L.dim + 64) * sizeof(float), e->stream, e->qbuf, (const S *)kpool,
                            (const S *)vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim,
-                           L.vdim, L.scale, L.sink, gate, ldg, (S *)out, ldo, v_row);
+                           L.vdim, L.scale, L.sink, gate, ldg, (S *)out, ldo, v_row, x.window, x.vshare, x.gate_per_head, x.out32);
         TL_CHECK_LAUNCH("hybrid attention");
         return TL_OK;
     }
-    if (dk4 <= 16 && vt_n <= 4) return launch_attn_tile<D, 16, 4>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
-    if (dk4 <= 32 && vt_n <= 8) return launch_attn_tile<D, 32, 8>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
-    if (vt_n <= 12) return launch_attn_tile<D, 64, 12>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);  // (a 192-wide latent beside a 64-wide rotated part)
-    return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
+    if (dk4 <= 16 && vt_n <= 4) return launch_attn_tile<D, 16, 4>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
+    if (dk4 <= 32 && vt_n <= 8) return launch_attn_tile<D, 32, 8>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
+    if (vt_n <= 12) return launch_attn_tile<D, 64, 12>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);  // (a 192-wide latent beside a 64-wide rotated part)
+    return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
 }
 
 static size_t attn_talk_lds(int es, int DK4, int VT, int G, int HGB) {
@@ -355,7 +377,7 @@ static int launch_attn_talk_tile(tl_hybrid *e, const tl_hybrid_layer &L, const v
     TL_CHECK_LAUNCH("hybrid attention tile (mixed heads)");
     if (sh.n_splits > 1) {
         hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
-                           ldg, (S *)out, ldo);
+                           ldg, (S *)out, ldo, 0, (float *)nullptr);
         TL_CHECK_LAUNCH("hybrid attention merge");
     }
     return TL_OK;
@@ -403,7 +425,7 @@ static int attention_talk(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
 
 static int launch_linrec(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
     const bool chan = L.rec_kind == TL_REC_CHANNEL;
-    const int ones = chan ? 0 : 1, VE = L.vdim + ones;
+    const int ones = L.rec_kind == TL_REC_EXPGATE ? 1 : 0, VE = L.vdim + ones;
     // lanes per state column: a wave while the step's columns are few (decode), a DPP row of 16 otherwise (or for narrow keys)
     const long cols = (long)L.heads * VE * n_seqs, simds = 4 * (long)qmm3_num_cus();
     int lpc = cols <= simds ? 64 : (cols <= 2 * simds + simds / 8 ? 32 : 16);
@@ -460,6 +482,26 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
     const int rows = sh.rows, n_seqs = sh.n_seqs, H = L.heads, HV = L.heads * L.vdim;
     if (L.kind == TL_MIX_ATTENTION) {
         const int G = L.kv_heads;
+        if (L.diff_maps || L.qk_head_norm || L.window > 0 || L.gated == 2) {
+            // q / k normed per head ahead of the rotation, maps side by side, a window on the keys, one gate per head
+            const int M = attn_maps(L);
+            hipLaunchKernelGGL((attn_prep_head_kernel<D>), dim3(rows, M * (H + G) + G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
+                               c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.rot_half, L.qk_head_norm, L.q_norm_dev, L.k_norm_dev, c.norm_eps,
+                               H, G, M, L.dim, L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+            TL_CHECK_LAUNCH("hybrid attention prep (per-head norm)");
+            const float *gate = L.gated ? e->proj + (size_t)M * (H + G) * L.dim + (size_t)G * L.vdim : nullptr;
+            AttnExtra x;
+            x.window = L.window, x.vshare = M, x.gate_per_head = L.gated == 2;
+            if (!L.diff_maps) return attention_core<D>(e, L, run.kpool, run.vpool, L.vdim, m, sh, gate, ldp, e->cat, ldcat, x);
+            tl_hybrid_layer A = L;  // every map is a head of its own over M * G K/V heads; the read-outs stay float32 for the combination
+            A.heads = M * H, A.kv_heads = M * G;
+            x.out32 = e->obuf;
+            HY_TRY(attention_core<D>(e, A, run.kpool, run.vpool, L.vdim, m, sh, nullptr, 0, nullptr, 0, x));
+            hipLaunchKernelGGL((diff_combine_kernel<D>), dim3(rows, H), dim3(64), 0, st, e->obuf, L.diff_lambda, L.diff_init, c.norm_eps, gate, ldp, x.gate_per_head, H, G,
+                               L.vdim, (S *)e->cat, ldcat);
+            TL_CHECK_LAUNCH("hybrid differential combination");
+            return TL_OK;
+        }
         if (L.qk_norm || L.rot_half || L.v_mix != TL_VMIX_NONE)  // (options of the row-wise preparation; create checked that it covers the layer)
             hipLaunchKernelGGL((attn_prep_row_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
                                c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.rot_half, L.qk_norm, L.q_norm_dev, L.k_norm_dev,
@@ -491,7 +533,7 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
         // ... and the values' onto the read-out: o_h = W_uv,h (sum_j p_j c_j)
         HY_TRY(linear_t<D>(e->da, H * L.kv_rank, L.uv_dev, e->obuf, HV, rows, L.vdim, L.kv_rank, 0, 1.f, nullptr, 0, st, H, L.kv_rank, (long)L.vdim * L.kv_rank, L.vdim));
         const size_t n = (size_t)rows * HV;
-        hipLaunchKernelGGL((gate_mul_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->obuf, HV, e->proj + g0, ldp, HV, 0, (S *)e->cat, ldcat, rows);
+        hipLaunchKernelGGL((gate_mul_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->obuf, HV, e->proj + g0, ldp, HV, L.gated ? 0 : 2, (S *)e->cat, ldcat, rows);
         TL_CHECK_LAUNCH("hybrid latent gate");
         return TL_OK;
     }
@@ -499,6 +541,16 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
         // proj: q (H dim) | k (H dim) | v (H vdim) | gate (H vdim) | i (H) | f (H)   or   ... | a1 (a_rank)
         const int g0 = 2 * H * L.dim + HV, x0 = g0 + HV;
         const bool chan = L.rec_kind == TL_REC_CHANNEL;
+        if (L.rec_kind == TL_REC_FIXED) {  // rotation of q and k, k * dim^-1/2, the constant decays as this step's gates
+            hipLaunchKernelGGL(fixed_decay_prep_kernel, dim3(rows, H), dim3(64), 0, st, e->proj, ldp, 0, H * L.dim, m.row_pos, e->inv_freq[run.layer], L.rot_dims,
+                               L.rot_half, 1.f / sqrtf((float)L.dim), L.decay_dev, e->gates, H, L.dim);
+            TL_CHECK_LAUNCH("hybrid constant decay prep");
+            HY_TRY(launch_linrec(e, L, run, m, n_seqs, ldp));
+            hipLaunchKernelGGL((linrec_out_kernel<D>), dim3(rows, H), dim3(64), 0, st, e->obuf, L.vdim, 0, e->gates, 1.f, L.out_norm_dev, 0, c.norm_eps, e->proj + g0, ldp,
+                               1, H, L.vdim, (S *)e->cat, ldcat);
+            TL_CHECK_LAUNCH("hybrid linrec out");
+            return TL_OK;
+        }
         if (chan) {
             const size_t na = (size_t)rows * L.a_rank, nd = (size_t)rows * H * L.dim;
             hipLaunchKernelGGL((cast_cols_kernel<D>), dim3((unsigned)((na + 255) / 256)), dim3(256), 0, st, e->proj, ldp, x0, L.a_rank, (S *)e->da, L.a_rank, rows);
@@ -577,7 +629,7 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
     hipStream_t st = e->stream;
     const int W = c.width;
     hipLaunchKernelGGL((embed_kernel<D>), dim3(rows), dim3(256), 0, st, m.tokens, (const S *)c.embed_dev, e->x0, e->x, W, c.vocab,
-                       c.embed_scale != 0.f ? c.embed_scale : 1.f);
+                       c.embed_scale != 0.f ? c.embed_scale : 1.f, c.embed_norm_dev, c.final_norm_offset, c.norm_eps);
     TL_CHECK_LAUNCH("hybrid embed");
     bool h_ready = false;  // e->h already holds this run's first norm (it left with the product that completed the previous residual sum)
     // the Dynamic Tanh norm that follows a residual sum: element-wise, so it can ride the completing product's epilogue
@@ -595,7 +647,11 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             const tl_hybrid_layer &Nx = e->layers[e->runs[ri + 1].layer];
             if (Nx.norm_kind == TL_NORM_DYT) next_first = tail_for(Nx.norm_dev, Nx.norm_bias_dev, Nx.norm_alpha);
         }
-        if (run.enters_pass) {  // x <- W_in [x ; x0] + step[pass]
+        if (run.enters_pass && !c.loop_in_dev) {  // x <- x + step[pass]
+            const size_t n = (size_t)rows * W;
+            hipLaunchKernelGGL(add_rowvec_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->x, c.loop_step_dev + (size_t)run.pass * W, W, rows);
+            TL_CHECK_LAUNCH("hybrid pass offset");
+        } else if (run.enters_pass) {  // x <- W_in [x ; x0] + step[pass]
             hipLaunchKernelGGL((pack2_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, e->x0, (S *)e->cat2, W);
             TL_CHECK_LAUNCH("hybrid pack2");
             HY_TRY(linear_t<D>(e->cat2, 2 * W, c.loop_in_dev, e->x, W, rows, W, 2 * W, 2, 1.f, c.loop_step_dev + (size_t)run.pass * W, 0, st));
@@ -651,7 +707,48 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
         }
         if (!h_ready) HY_TRY(norm_t<D>(e, L.norm_kind, L.norm_dev, L.norm_bias_dev, L.norm_alpha, L.norm_offset, e->h, nullptr, rows));
         h_ready = false;
-        if (c.parallel_block == TL_BLOCK_PARALLEL) {
+        if (c.parallel_block == TL_BLOCK_SANDWICH) {
+            // x += m ls1 post1(W_o mixer(norm1 x));  x += m ls2 post2(ff(norm2 x));  x += side(x).  Each sum's kernel also writes what reads the new
+            // stream next: the feed-forward's norm, the stream itself for the token input, or the next run's first norm.
+            const tl_hybrid_layer *Nx = (ri + 1 < e->runs.size() && !e->runs[ri + 1].enters_pass) ? &e->layers[e->runs[ri + 1].layer] : nullptr;
+            const bool side = L.side_gate_dev != nullptr;
+            const int threads = rows < 64 ? 1024 : 256;
+            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, L.w_in_bias_dev ? 2 : 0, 1.f, L.w_in_bias_dev, 0, st));
+            HY_TRY(mixer_t<D>(e, ri, m, sh, nmix, HV));
+            HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->y, W, rows, W, HV, 0, 1.f, nullptr, 0, st));
+            {
+                const int next = L.ff > 0 ? 2 : (side ? 1 : (Nx ? 2 : 0));
+                const float *nw = L.ff > 0 ? L.norm2_dev : (Nx ? Nx->norm_dev : nullptr);
+                hipLaunchKernelGGL((sandwich_add_kernel<D>), dim3(rows), dim3(threads), 0, st, e->x, e->y, L.post_norm_dev, L.norm_offset, c.norm_eps, c.residual_mult,
+                                   L.ls1_dev, next, nw, L.ff > 0 ? L.norm_offset : (Nx ? Nx->norm_offset : 0.f), (S *)e->h, W);
+                TL_CHECK_LAUNCH("hybrid norm on the mixer's output");
+                h_ready = L.ff <= 0 && !side && next == 2;
+            }
+            if (L.ff > 0) {
+                const int nin2 = ff_in_cols(L);
+                HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
+                HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
+                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->y, W, rows, W, L.ff, 0, 1.f, nullptr, 0, st));
+                const int next = side ? 1 : (Nx ? 2 : 0);
+                hipLaunchKernelGGL((sandwich_add_kernel<D>), dim3(rows), dim3(threads), 0, st, e->x, e->y, L.post_norm2_dev, L.norm_offset, c.norm_eps, c.residual_mult,
+                                   L.ls2_dev, next, Nx ? Nx->norm_dev : nullptr, Nx ? Nx->norm_offset : 0.f, (S *)e->h, W);
+                TL_CHECK_LAUNCH("hybrid norm on the feed-forward's output");
+                h_ready = !side && next == 2;
+            }
+            if (side) {  // y = W_proj (gelu_tanh(W_gate x) * e);  x += y / rms(y) * side_norm
+                const int sd = c.side_dim;
+                HY_TRY(linear_t<D>(e->h, W, L.side_gate_dev, e->proj, sd, rows, sd, W, 0, 1.f, nullptr, 0, st));
+                const size_t n = (size_t)rows * sd;
+                hipLaunchKernelGGL((side_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, sd, m.tokens, (const S *)c.side_embed_dev, c.side_cols,
+                                   L.side_col0, sd, c.vocab, (S *)e->cat, sd, rows);
+                TL_CHECK_LAUNCH("hybrid token input");
+                HY_TRY(linear_t<D>(e->cat, sd, L.side_proj_dev, e->y, W, rows, W, sd, 0, 1.f, nullptr, 0, st));
+                hipLaunchKernelGGL((sandwich_add_kernel<D>), dim3(rows), dim3(threads), 0, st, e->x, e->y, L.side_norm_dev, 0.f, c.norm_eps, 1.f, (const float *)nullptr,
+                                   Nx ? 2 : 0, Nx ? Nx->norm_dev : nullptr, Nx ? Nx->norm_offset : 0.f, (S *)e->h, W);
+                TL_CHECK_LAUNCH("hybrid norm on the token input");
+                h_ready = Nx != nullptr;
+            }
+        } else if (c.parallel_block == TL_BLOCK_PARALLEL) {
             const int nin = nmix + L.ff, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
             HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nin, rows, nin, W, 0, 1.f, nullptr, 0, st));
             HY_TRY(mixer_t<D>(e, ri, m, sh, nin, ldcat));
@@ -761,14 +858,16 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     const tl_hybrid_config &c = *cfg;
     TL_REQUIRE(c.dtype == TL_HY_BF16 || c.dtype == TL_HY_F32, "hybrid_create: dtype must be bfloat16 or float32");
     TL_REQUIRE(c.width > 0 && c.vocab > 0 && c.num_layers > 0, "hybrid_create: width, vocab and num_layers must be positive");
-    TL_REQUIRE(c.parallel_block >= 0 && c.parallel_block <= 2, "hybrid_create: parallel_block is 0 (sequential), 1 (parallel) or 2 (norm on the branch's output)");
+    TL_REQUIRE(c.parallel_block >= 0 && c.parallel_block <= 3,
+               "hybrid_create: parallel_block is 0 (sequential), 1 (parallel), 2 (norm on the branch's output) or 3 (norms on both sides)");
+    TL_REQUIRE(c.side_dim >= 0 && (c.side_dim == 0 || (c.side_embed_dev && c.side_cols >= c.side_dim)), "hybrid_create: a token-input table needs its width");
     TL_REQUIRE(c.final_norm_kind == TL_NORM_RMS || (c.final_norm_kind == TL_NORM_DYT && c.final_norm_bias_dev), "hybrid_create: final norm kind");
     TL_REQUIRE(c.page_size > 0 && c.num_pages > 0 && c.max_slots > 0 && c.max_pages_per_seq > 0 && c.max_rows > 0, "hybrid_create: pool sizes must be positive");
     TL_REQUIRE(c.embed_dev && c.final_norm_dev && c.head_dev, "hybrid_create: embed, final norm and head are required");
     const bool looped = c.loop_times > 1 || (c.loop_times == 1 && c.loop_stop > c.loop_start);
     if (looped) {
         TL_REQUIRE(c.loop_start >= 0 && c.loop_stop > c.loop_start && c.loop_stop <= c.num_layers, "hybrid_create: loop range outside the layer list");
-        TL_REQUIRE(c.loop_in_dev && c.loop_step_dev, "hybrid_create: a loop needs its entry projection and pass offsets");
+        TL_REQUIRE(c.loop_step_dev, "hybrid_create: a loop needs its pass offsets");
     }
     auto e = std::make_unique<tl_hybrid>();
     e->cfg = c;
@@ -789,6 +888,15 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         TL_REQUIRE(L.norm_kind == TL_NORM_RMS || (L.norm_kind == TL_NORM_DYT && L.norm_bias_dev), "hybrid_create: norm kind (Dynamic Tanh needs its bias)");
         if (c.parallel_block == TL_BLOCK_POSTNORM)
             TL_REQUIRE(L.norm_kind == TL_NORM_RMS && !L.ls1_dev && !L.ls2_dev && !looped, "hybrid_create: the block with the norm on the branch's output takes RMS norms, no layer scale and no loop");
+        if (c.parallel_block == TL_BLOCK_SANDWICH) {
+            TL_REQUIRE(L.norm_kind == TL_NORM_RMS && L.post_norm_dev && (L.ff <= 0 || L.post_norm2_dev), "hybrid_create: the block with norms on both sides takes RMS norms and a weight for every branch's result");
+            TL_REQUIRE(L.ff <= 0 || L.ff_kind == TL_FF_PLAIN || L.ff_kind == TL_FF_GATED, "hybrid_create: the block with norms on both sides takes a dense feed-forward");
+        }
+        TL_REQUIRE((!L.side_gate_dev && !L.side_proj_dev && !L.side_norm_dev) ||
+                       (c.parallel_block == TL_BLOCK_SANDWICH && L.side_gate_dev && L.side_proj_dev && L.side_norm_dev && c.side_dim > 0 && L.side_col0 >= 0 &&
+                        L.side_col0 + c.side_dim <= c.side_cols),
+                   "hybrid_create: a per-layer token input needs its three tensors, the table, and the block with norms on both sides");
+        TL_REQUIRE(!L.w_in_bias_dev || c.parallel_block == TL_BLOCK_SANDWICH, "hybrid_create: projection biases are read by the block with norms on both sides only");
         if (c.parallel_block == TL_BLOCK_PARALLEL) {
             TL_REQUIRE(L.ff_kind == TL_FF_PLAIN && !L.ls1_dev && !L.ls2_dev, "hybrid_create: the parallel block takes a plain feed-forward and no layer scale");
         } else if (L.ff > 0) {
@@ -813,6 +921,14 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
             TL_REQUIRE(!(L.qk_unit_rms && (L.qk_norm || L.rot_half || L.v_mix != TL_VMIX_NONE)),
                        "hybrid_create: unit-RMS heads after the rotation do not combine with the whole-projection norm, half-split rotation pairs or value mixing");
             TL_REQUIRE(L.chunk >= 0 && L.v_mix >= TL_VMIX_NONE && L.v_mix <= TL_VMIX_BLEND, "hybrid_create: chunk >= 0, v_mix 0..2");
+            TL_REQUIRE(L.gated >= 0 && L.gated <= 2 && L.window >= 0, "hybrid_create: gated 0..2, window >= 0");
+            if (L.diff_maps || L.qk_head_norm || L.window > 0 || L.gated == 2) {
+                TL_REQUIRE(!L.qk_unit_rms && !L.qk_norm && L.v_mix == TL_VMIX_NONE && !L.talk_dev && !L.sink_dev && L.chunk == 0,
+                           "hybrid_create: per-head norms, maps, a window and per-head gates do not combine with unit-RMS heads, the whole-projection norm, value mixing, "
+                           "mixed scores, learned sinks or a chunked mask");
+                TL_REQUIRE(!L.qk_head_norm || (L.q_norm_dev && L.k_norm_dev), "hybrid_create: a norm per head needs its weights");
+                TL_REQUIRE(!L.diff_maps || !L.sink, "hybrid_create: differential attention takes no sink");
+            }
             if (L.v_mix != TL_VMIX_NONE) {
                 if (vmix_width == 0) {
                     TL_REQUIRE(L.v_mix == TL_VMIX_FIRST, "hybrid_create: the first value-mixing layer keeps its values (v_mix 1), later ones blend (v_mix 2)");
@@ -821,8 +937,10 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
                     TL_REQUIRE(L.v_mix == TL_VMIX_BLEND && L.kv_heads * L.vdim == vmix_width, "hybrid_create: value-mixing layers share one values width");
             }
         } else if (L.kind == TL_MIX_LINREC) {
-            TL_REQUIRE(L.kv_heads == L.heads && L.out_norm_dev, "hybrid_create: a linear recurrence has one key head per head and an output norm weight");
-            if (L.rec_kind == TL_REC_CHANNEL)
+            TL_REQUIRE(L.kv_heads == L.heads && (L.out_norm_dev || L.rec_kind == TL_REC_FIXED), "hybrid_create: a linear recurrence has one key head per head and an output norm weight");
+            if (L.rec_kind == TL_REC_FIXED)
+                TL_REQUIRE(L.decay_dev && L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.dim, "hybrid_create: a constant decay needs its values; rot_dims even and at most dim");
+            else if (L.rec_kind == TL_REC_CHANNEL)
                 TL_REQUIRE(L.a_rank >= 1 && L.a2_dev && L.a2_bias_dev && L.tau > 0.f, "hybrid_create: channel decay needs its projection pair, bias and tau > 0");
             else
                 TL_REQUIRE(L.rec_kind == TL_REC_EXPGATE && L.i_bias_dev && L.f_bias_dev && L.gate_cap > 0.f, "hybrid_create: exponential gates need biases and a cap > 0");
@@ -846,9 +964,10 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         const bool par = c.parallel_block == TL_BLOCK_PARALLEL;
         max_in = std::max(max_in, par ? mixer_cols(L) + L.ff : std::max(mixer_cols(L), ff_in_cols(L)));
         max_cat = std::max(max_cat, par ? L.heads * L.vdim + L.ff : std::max(L.heads * L.vdim, L.ff));
-        max_hv = std::max(max_hv, L.heads * (L.vdim + 1));
+        max_hv = std::max(max_hv, attn_maps(L) * L.heads * (L.vdim + 1));
         max_gh = std::max(max_gh, L.heads);
-        if (L.kind == TL_MIX_ATTENTION) max_q = std::max(max_q, L.heads * L.dim);
+        if (L.side_gate_dev) max_in = std::max(max_in, c.side_dim), max_cat = std::max(max_cat, c.side_dim);
+        if (L.kind == TL_MIX_ATTENTION) max_q = std::max(max_q, attn_maps(L) * L.heads * L.dim);
         else if (L.kind == TL_MIX_LATENT) {
             max_q = std::max(max_q, L.heads * (L.kv_rank + L.rot_dim));
             max_c = std::max(max_c, L.heads * (L.dim + L.rot_dim));
@@ -883,7 +1002,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     e->rot_mult.assign(c.num_layers, 1.f);
     for (int i = 0; i < c.num_layers; ++i) {
         const tl_hybrid_layer &L = e->layers[i];
-        if (L.kind != TL_MIX_ATTENTION && L.kind != TL_MIX_LATENT) continue;
+        if (L.kind != TL_MIX_ATTENTION && L.kind != TL_MIX_LATENT && !(L.kind == TL_MIX_LINREC && L.rec_kind == TL_REC_FIXED)) continue;
         const int half = std::max(1, L.rot_dims / 2);
         std::vector<float> f(half, 0.f);
         for (int k = 0; k < L.rot_dims / 2; ++k) f[k] = (float)std::pow((double)L.rot_base, -2.0 * k / (double)L.rot_dims);
@@ -938,7 +1057,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
             HY_TRY(dev_alloc(p, &r.conv_state, mb, true));
             e->stats.state_bytes += (sb + mb) * 4;
         } else if (L.kind == TL_MIX_ATTENTION) {
-            const size_t kb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.dim * es, vb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.vdim * es;
+            const size_t kb = (size_t)c.num_pages * attn_maps(L) * L.kv_heads * c.page_size * L.dim * es, vb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.vdim * es;
             HY_TRY(dev_alloc(p, (char **)&r.kpool, kb, true));
             HY_TRY(dev_alloc(p, (char **)&r.vpool, vb, true));
             e->stats.kv_bytes += kb + vb;
@@ -958,7 +1077,8 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     if (c.parallel_block == TL_BLOCK_POSTNORM) {
         HY_TRY(dev_alloc(p, &e->y, (size_t)R * W));
         HY_TRY(dev_alloc(p, &e->moe_mask, 1, true));
-    }
+    } else if (c.parallel_block == TL_BLOCK_SANDWICH)
+        HY_TRY(dev_alloc(p, &e->y, (size_t)R * W));
     if (vmix_width > 0) HY_TRY(dev_alloc(p, &e->vref, (size_t)R * vmix_width));
     HY_TRY(dev_alloc(p, &e->proj, (size_t)R * e->ld_proj));
     HY_TRY(dev_alloc(p, &e->qbuf, (size_t)R * std::max(1, max_q)));
@@ -971,7 +1091,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     HY_TRY(dev_alloc(p, &e->logits, (size_t)R * c.vocab));
     int max_h = 1, max_v = 1;
     for (const tl_hybrid_layer &L : e->layers)
-        if (L.kind == TL_MIX_ATTENTION) max_h = std::max(max_h, L.heads), max_v = std::max(max_v, L.vdim);
+        if (L.kind == TL_MIX_ATTENTION) max_h = std::max(max_h, attn_maps(L) * L.heads), max_v = std::max(max_v, L.vdim);
         else if (L.kind == TL_MIX_LATENT) max_h = std::max(max_h, L.heads), max_v = std::max(max_v, L.kv_rank);
     HY_TRY(dev_alloc(p, &e->part_acc, (size_t)c.max_slots * max_h * 64 * max_v));
     HY_TRY(dev_alloc(p, &e->part_ml, (size_t)c.max_slots * max_h * 64 * 2));

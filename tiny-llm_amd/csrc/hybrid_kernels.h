@@ -34,14 +34,27 @@ __device__ __forceinline__ float act_f(float z, int kind) {
     return silu_f(z);
 }
 
-// ---- embedding gather: x0 = x = embed[token] * scale -----------------------------------------------------------
+// ---- embedding gather: x0 = x = embed[token] * scale; with nw the row then passes an RMS norm, * (noffset + nw) ------
 template <typename D>
-__global__ void embed_kernel(const int32_t *tokens, const typename D::storage *embed, float *x0, float *x, int width, int vocab, float scale) {
+__global__ void embed_kernel(const int32_t *tokens, const typename D::storage *embed, float *x0, float *x, int width, int vocab, float scale,
+                             const float *nw, float noffset, float eps) {
+    __shared__ float red[16];
     const int t = blockIdx.x;
     int tok = tokens[t];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    float inv = 1.f;
+    if (nw) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < width; c += blockDim.x) {
+            const float v = ld<D>(embed, (size_t)tok * width + c) * scale;
+            ss += v * v;
+        }
+        ss = block_sum(ss, red);
+        inv = 1.f / sqrtf(ss / (float)width + eps);
+    }
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = ld<D>(embed, (size_t)tok * width + c) * scale;
+        float v = ld<D>(embed, (size_t)tok * width + c) * scale;
+        if (nw) v = v * inv * (noffset + nw[c]);
         x0[(size_t)t * width + c] = v;
         x[(size_t)t * width + c] = v;
     }
@@ -350,18 +363,21 @@ template <typename D>
 __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
                                                        const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
                                                        const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
-                                                       float scale, int sink, const float *gate, int ldg, typename D::storage *out, int ldo, int v_row) {
+                                                       float scale, int sink, const float *gate, int ldg, typename D::storage *out, int ldo, int v_row,
+                                                       int window, int vshare, int gate_per_head, float *out32) {
     extern __shared__ float smem[];
     float *qs = smem;        // [dim]
     float *ps = smem + dim;  // [64]
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int pos = row_pos[t], slot = seq_slot[row_seq[t]], g = h / (H / G);
+    // window > 0: the keys start window - 1 positions before the query.  vshare K/V heads in a row read one value head.
+    const int Gv = G / vshare, gv = g / vshare, k_lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int32_t *bt = block_table + (size_t)slot * max_pages;
     for (int c = lane; c < dim; c += 64) qs[c] = qbuf[((size_t)t * H + h) * dim + c];
     __syncthreads();
     float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // vdim <= 512
-    for (int kb = 0; kb <= pos; kb += 64) {
+    for (int kb = k_lo; kb <= pos; kb += 64) {
         const int j = kb + lane;
         float s = -INFINITY;
         if (j <= pos) {
@@ -383,7 +399,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
         for (int i = 0; i < 8; ++i) acc[i] *= corr;
         for (int jj = 0; jj < cnt; ++jj) {
             const int jg = kb + jj;
-            const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + g) * page_size + jg % page_size) * v_row;
+            const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * Gv + gv) * page_size + jg % page_size) * v_row;
             const float pj = ps[jj];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -398,8 +414,9 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
         const int c = lane + i * 64;
         if (c < vdim) {
             float o = acc[i] * invl;
-            if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]);
-            out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o);
+            if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + (gate_per_head ? (size_t)h : (size_t)h * vdim + c)]);
+            if (out32) out32[((size_t)t * H + h) * vdim + c] = o;
+            else out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o);
         }
     }
 }
@@ -420,9 +437,12 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                                                         const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
                                                         float scale, int sink, int HGB, int n_hblk, int keys_per_split, int n_splits, const float *gate,
                                                         int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml, int page_shift,
-                                                        int vec_ok, int v_row) {
+                                                        int vec_ok, int v_row, int window, int vshare, int gate_per_head, float *out32) {
     using S = typename D::storage;
     extern __shared__ float smem[];
+    // window > 0: a query sees key j <= its position only if position - j < window; the walk starts at the first key the tile's first row sees,
+    // and a split key range (decode steps) is counted from there.  vshare: that many K/V heads in a row read one value head (maps over shared
+    // values).  out32: the read-out as float32 rows [row, head, vdim] instead of D rows of `out` (no gate).
     // LDS rows as wide as the template: zeros behind dim / vdim, no guards in the product loops.  bfloat16 pages: the K tile stays bfloat16
     // in LDS ([64][4 DK4 + 8] 16-bit elements) and S^T runs on v_mfma_f32_16x16x32_bf16 (q rounded to bfloat16 like every other input of a
     // bfloat16 product, float32 sums, the scale applied to the float32 result); the weights and P V are float32 in either case.
@@ -438,7 +458,9 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
     const int pos0 = row_pos[r0], slot = seq_slot[seq];
     const int32_t *bt = block_table + (size_t)slot * max_pages;
     const int k_end_tile = pos0 + min(t0 + TQ, len);  // keys the tile's last query row sees
-    const int k_begin = split * keys_per_split, k_end = min(k_end_tile, (split + 1) * keys_per_split);
+    const int k_lo = window > 0 ? max(0, pos0 + t0 - window + 1) : 0;
+    const int k_begin = k_lo + split * keys_per_split, k_end = min(k_end_tile, k_lo + (split + 1) * keys_per_split);
+    const int Gv = G / vshare, kvh_v = kvh / vshare;
     // this lane's query row (column of the transposed products)
     // WSPLIT (a tile with at most 16 query rows, i.e. decode steps): every wave holds the SAME 16 rows and takes the 16 keys `wave` of each
     // 64-key tile -- a quarter of the products per wave -- and the four partial (max, sum, O) sets are merged through LDS at the end
@@ -496,7 +518,8 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                 if (pl >= 0 && j < k_end && c8 < (is_v ? vdim : dim)) {
                     const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
                     const int wd = is_v ? vdim : dim;  // v_row: the width of a row of vpool (vdim, or the key row's when the values are its leading columns)
-                    const S *src = (is_v ? vpool : kpool) + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * (is_v ? v_row : dim) + c8;
+                    const S *src = (is_v ? vpool + (((size_t)bt[pg] * Gv + kvh_v) * page_size + in_pg) * v_row
+                                         : kpool + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * dim) + c8;
                     if (vec_ok) {  // (widths are multiples of 8: a chunk is whole or absent)
                         if constexpr (sizeof(S) == 2) *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
                         else {
@@ -563,7 +586,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * n + 4 * g4 + r;
-                    a4[r] = (row_ok && j <= qpos && j < k_end) ? a4[r] : -INFINITY;
+                    a4[r] = (row_ok && j <= qpos && j < k_end && (window <= 0 || qpos - j < window)) ? a4[r] : -INFINITY;
                     m_tile = fmaxf(m_tile, a4[r]);
                 }
                 sc[nn] = a4;
@@ -643,8 +666,9 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                 const int c = 16 * v + 4 * g4 + r;
                 if (c < vdim) {
                     float val = o[v][r] * invl;
-                    if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (size_t)head * vdim + c]);
-                    out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
+                    if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (gate_per_head ? (size_t)head : (size_t)head * vdim + c)]);
+                    if (out32) out32[((size_t)trow * H + head) * vdim + c] = val;
+                    else out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
                 }
             }
     } else {
@@ -667,7 +691,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 // sum and the weights exp(m_s - M); then the lanes turn to the value columns and walk the splits with those weights.
 template <typename D>
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, int H, int vdim, const float *gate,
-                                                        int ldg, typename D::storage *out, int ldo) {
+                                                        int ldg, typename D::storage *out, int ldo, int gate_per_head, float *out32) {
     __shared__ float ws[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const size_t p0 = ((size_t)t * H + h) * n_splits;
@@ -684,8 +708,99 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, c
 #pragma unroll 8
         for (int s = 0; s < n_splits; ++s) acc += part_acc[(p0 + s) * vdim + c] * ws[s];
         float val = acc * invl;
-        if (gate) val *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]);
-        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(val);
+        if (gate) val *= sigmoid_f(gate[(size_t)t * ldg + (gate_per_head ? (size_t)h : (size_t)h * vdim + c)]);
+        if (out32) out32[((size_t)t * H + h) * vdim + c] = val;
+        else out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(val);
+    }
+}
+
+// ---- attention, step 1 (head form with a norm ahead of the rotation): one wave per (row, head and map of q | k, value head) ------------------
+// proj: q | k | v at columns 0 | H*M*dim | (H+G)*M*dim; M maps per head lie side by side ([map 1 | map 2] with M = 2).  Every (head, map) of q and
+// k: x / sqrt(mean x^2 + eps) * w over dim (qw / kw [dim], shared by all heads and maps; head_norm 0: none), then the rotation of the first
+// rot_dims dimensions by pos * inv_freq[i]: pairs (i, i + rot_dims/2) with rot_half, (2i, 2i+1) without.
+// q goes to qbuf as H*M heads ordered [K/V head][map][head in group], k to kpool as G*M K/V heads [K/V head][map]: query head e of that order reads
+// K/V head e / (H/G), and K/V head g reads value head g / M.
+template <typename D>
+__global__ __launch_bounds__(64) void attn_prep_head_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
+                                                            const int32_t *block_table, int max_pages, int page_size, const float *inv_freq, int rot_dims,
+                                                            int rot_half, int head_norm, const float *qw, const float *kw, float eps, int H, int G, int M, int dim,
+                                                            int vdim, float *qbuf, typename D::storage *kpool, typename D::storage *vpool) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[t], slot = seq_slot[row_seq[t]];
+    const int page = block_table[(size_t)slot * max_pages + pos / page_size], in_page = pos % page_size;
+    const int HM = H * M, GM = G * M;
+    if (hh >= HM + GM) {  // a value head: copy
+        const int g = hh - HM - GM;
+        const float *src = proj + (size_t)t * ldp + (size_t)(HM + GM) * dim + (size_t)g * vdim;
+        typename D::storage *dst = vpool + (((size_t)page * G + g) * page_size + in_page) * vdim;
+        for (int c = lane; c < vdim; c += 64) dst[c] = D::from_float(src[c]);
+        return;
+    }
+    const bool is_q = hh < HM;
+    const float *src = proj + (size_t)t * ldp + (size_t)hh * dim;
+    const float *w = head_norm ? (is_q ? qw : kw) : nullptr;
+    float inv = 1.f;
+    if (head_norm) {
+        float ss = 0.f;
+        for (int c = lane; c < dim; c += 64) ss += src[c] * src[c];
+        ss = wave_sum(ss);
+        inv = 1.f / sqrtf(ss / (float)dim + eps);
+    }
+    float *qdst = nullptr;
+    typename D::storage *kdst = nullptr;
+    if (is_q) {
+        const int h = hh / M, mp = hh % M, HG = H / G;
+        qdst = qbuf + ((size_t)t * HM + ((size_t)(h / HG) * M + mp) * HG + h % HG) * dim;
+    } else
+        kdst = kpool + (((size_t)page * GM + (hh - HM)) * page_size + in_page) * dim;
+    const int half = rot_dims / 2, units = dim - half;  // `half` rotation pairs, then the dimensions that pass
+    for (int u = lane; u < units; u += 64) {
+        int c0, c1 = -1;
+        if (u < half) c0 = rot_half ? u : 2 * u, c1 = rot_half ? u + half : 2 * u + 1;
+        else c0 = u + half;
+        float a = src[c0] * inv * (w ? w[c0] : 1.f), b2 = 0.f;
+        if (c1 >= 0) {
+            b2 = src[c1] * inv * (w ? w[c1] : 1.f);
+            float sn, cs;
+            sincosf((float)pos * inv_freq[u], &sn, &cs);
+            const float na = a * cs - b2 * sn, nb = b2 * cs + a * sn;
+            a = na, b2 = nb;
+        }
+        if (is_q) {
+            qdst[c0] = a;
+            if (c1 >= 0) qdst[c1] = b2;
+        } else {
+            kdst[c0] = D::from_float(a);
+            if (c1 >= 0) kdst[c1] = D::from_float(b2);
+        }
+    }
+}
+
+// ---- differential attention, last step: one wave per (row, head).  a [rows, H*2, vdim] float32 in the order attn_prep_head_kernel gives the
+// maps ([K/V head][map][head in group]); o = a1 - lambda a2;  o / sqrt(mean o^2 + eps) * (1 - init) * sigmoid(gate) -> D rows.
+// gate (may be NULL): one number per head (gate_per_head) or per output channel.
+template <typename D>
+__global__ __launch_bounds__(64) void diff_combine_kernel(const float *a, float lambda, float init, float eps, const float *gate, int ldg, int gate_per_head,
+                                                          int H, int G, int vdim, typename D::storage *out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, HG = H / G;
+    const float *a1 = a + ((size_t)t * 2 * H + ((size_t)(h / HG) * 2) * HG + h % HG) * vdim, *a2 = a1 + (size_t)HG * vdim;
+    float o[8], ss = 0.f;  // vdim <= 512
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = lane + 64 * i;
+        o[i] = c < vdim ? a1[c] - lambda * a2[c] : 0.f;
+        ss += o[i] * o[i];
+    }
+    ss = wave_sum(ss);
+    const float mul = (1.f - init) / sqrtf(ss / (float)vdim + eps);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = lane + 64 * i;
+        if (c < vdim) {
+            float v = o[i] * mul;
+            if (gate) v *= sigmoid_f(gate[(size_t)t * ldg + (gate_per_head ? (size_t)h : (size_t)h * vdim + c)]);
+            out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(v);
+        }
     }
 }
 
@@ -1214,6 +1329,42 @@ __global__ void postnorm_add_kernel(float *x, const float *y, const float *w, fl
         h[(size_t)r * width + c] = D::from_float(v);
     }
 }
+// ---- the block with norms on both sides: x += mult * ls * (y / sqrt(mean y^2 + eps) * (offset + w))  (ls NULL: 1), and what reads the new
+// stream next leaves with it: next 1: h = x as D rows;  next 2: h = x / sqrt(mean x^2 + eps) * (noffset + nw) as D rows;  0: nothing ----
+template <typename D>
+__global__ void sandwich_add_kernel(float *x, const float *y, const float *w, float offset, float eps, float mult, const float *ls, int next,
+                                    const float *nw, float noffset, typename D::storage *h, int width) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const float *src = y + (size_t)r * width;
+    float *xr = x + (size_t)r * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) ss += src[c] * src[c];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+    float s2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = xr[c] + mult * (ls ? ls[c] : 1.f) * (src[c] * inv * (offset + w[c]));
+        xr[c] = v;
+        s2 += v * v;
+        if (next == 1) h[(size_t)r * width + c] = D::from_float(v);
+    }
+    if (next != 2) return;
+    s2 = block_sum(s2, red);
+    const float inv2 = 1.f / sqrtf(s2 / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) h[(size_t)r * width + c] = D::from_float(xr[c] * inv2 * (noffset + nw[c]));  // (this thread's own writes)
+}
+// per-layer token input, middle step: cat[t, c] = gelu_tanh(proj[t, c]) * table[token[t], col0 + c], c < n
+template <typename D>
+__global__ void side_act_kernel(const float *proj, int ldp, const int32_t *tokens, const typename D::storage *table, int table_cols, int col0, int n, int vocab,
+                                typename D::storage *out, int ldo, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * n) return;
+    const int t = (int)(i / n), c = (int)(i % n);
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    out[(size_t)t * ldo + c] = D::from_float(act_f(proj[(size_t)t * ldp + c], 1) * ld<D>(table, (size_t)tok * table_cols + col0 + c));
+}
 // float32 rows -> D rows (the input of a sublayer that reads the stream itself)
 template <typename D>
 __global__ void cast_rows_kernel(const float *x, typename D::storage *out, size_t n) {
@@ -1512,14 +1663,14 @@ __global__ __launch_bounds__(64) void latent_prep_kernel(const float *q, int H, 
     }
 }
 
-// ---- out[t, c] = in[t, c] * gate(g[t, c]) as D rows.  kind 0: sigmoid, 1: SiLU ----------------------------------------------------
+// ---- out[t, c] = in[t, c] * gate(g[t, c]) as D rows.  kind 0: sigmoid, 1: SiLU, 2: no gate (g is not read) ----------------------------
 template <typename D>
 __global__ void gate_mul_kernel(const float *in, int ldi, const float *g, int ldg, int n, int kind, typename D::storage *out, int ldo, int rows) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)rows * n) return;
     const int t = (int)(i / n), c = (int)(i % n);
-    const float z = g[(size_t)t * ldg + c];
-    out[(size_t)t * ldo + c] = D::from_float(in[(size_t)t * ldi + c] * (kind == 0 ? sigmoid_f(z) : silu_f(z)));
+    const float z = kind == 2 ? 0.f : g[(size_t)t * ldg + c];
+    out[(size_t)t * ldo + c] = D::from_float(in[(size_t)t * ldi + c] * (kind == 2 ? 1.f : (kind == 0 ? sigmoid_f(z) : silu_f(z))));
 }
 
 // ---- gated feed-forward activation: cat[t, col0 + c] = act(proj[t, g0 + c]) * proj[t, u0 + c] ------------------------------------
@@ -1714,6 +1865,31 @@ __global__ __launch_bounds__(256) void linrec_kernel(const float *proj, int ldp,
     }
 }
 
+// Constant decay per head (retention), ahead of the recurrence: q and k of every (row, head) turn in place (float32 columns q0 / k0 of proj) on their
+// first rot_dims dimensions by pos * inv_freq[i] -- pairs (i, i + rot_dims/2) with rot_half, (2i, 2i+1) without -- then k is multiplied by k_scale;
+// gates[t, h] = (decay[h], 1, -).  One wave per (row, head).
+__global__ __launch_bounds__(64) void fixed_decay_prep_kernel(float *proj, int ldp, int q0, int k0, const int32_t *row_pos, const float *inv_freq, int rot_dims,
+                                                              int rot_half, float k_scale, const float *decay, float *gates, int H, int dim) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[t], half = rot_dims / 2;
+    float *q = proj + (size_t)t * ldp + q0 + (size_t)h * dim, *k = proj + (size_t)t * ldp + k0 + (size_t)h * dim;
+    for (int u = lane; u < dim - half; u += 64) {
+        if (u < half) {
+            const int c0 = rot_half ? u : 2 * u, c1 = rot_half ? u + half : 2 * u + 1;
+            float sn, cs;
+            sincosf((float)pos * inv_freq[u], &sn, &cs);
+            const float qa = q[c0], qb = q[c1], ka = k[c0], kb = k[c1];
+            q[c0] = qa * cs - qb * sn, q[c1] = qb * cs + qa * sn;
+            k[c0] = (ka * cs - kb * sn) * k_scale, k[c1] = (kb * cs + ka * sn) * k_scale;
+        } else
+            k[u + half] *= k_scale;
+    }
+    if (lane == 0) {
+        float *g = gates + ((size_t)t * H + h) * 3;
+        g[0] = decay[h], g[1] = 1.f, g[2] = 0.f;
+    }
+}
+
 // read-out of a linear recurrence, one wave per (row, head):  o = obuf[t, h, :vdim] * qscale;  with ones: o /= max(|n.q|, e) + 1e-6 where n.q is
 // the appended column (times qscale) and e the gate floor;  then o / rms(o) * w[h * w_stride + c] * gate(g)   (gate_kind 0 sigmoid, 1 SiLU)
 template <typename D>
@@ -1733,7 +1909,7 @@ __global__ __launch_bounds__(64) void linrec_out_kernel(const float *obuf, int V
     const float inv = mul / sqrtf(ss / (float)vdim + eps);
     for (int c = lane; c < vdim; c += 64) {
         const float z = gate[(size_t)t * ldg + (size_t)h * vdim + c];
-        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o[c] * inv * w[(size_t)h * w_stride + c] * (gate_kind == 0 ? sigmoid_f(z) : silu_f(z)));
+        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o[c] * inv * (w ? w[(size_t)h * w_stride + c] : 1.f) * (gate_kind == 0 ? sigmoid_f(z) : silu_f(z)));
     }
 }
 

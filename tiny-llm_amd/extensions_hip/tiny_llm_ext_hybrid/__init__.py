@@ -23,11 +23,11 @@ _vp, _i, _f, _sz, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_s
 _P = ctypes.POINTER
 
 MIX_ATTENTION, MIX_DELTA, MIX_LINREC, MIX_LATENT = 0, 1, 2, 3
-REC_CHANNEL, REC_EXPGATE = 0, 1
+REC_CHANNEL, REC_EXPGATE, REC_FIXED = 0, 1, 2
 NORM_RMS, NORM_DYT = 0, 1
 FF_PLAIN, FF_GATED, FF_MOE = 0, 1, 2
 ROUTER_SOFTMAX, ROUTER_SIGMOID = 0, 1
-BLOCK_SEQUENTIAL, BLOCK_PARALLEL, BLOCK_POSTNORM = 0, 1, 2
+BLOCK_SEQUENTIAL, BLOCK_PARALLEL, BLOCK_POSTNORM, BLOCK_SANDWICH = 0, 1, 2, 3
 VMIX_NONE, VMIX_FIRST, VMIX_BLEND = 0, 1, 2
 HY_F32, HY_BF16 = 0, 2
 FF_GELU_ERF, FF_GELU_TANH, FF_SILU, FF_RELU2 = 0, 1, 2, 3
@@ -50,7 +50,10 @@ class TlHybridLayer(ctypes.Structure):
                 ("rot_factor", _f), ("rot_original", _f), ("rot_fast", _f), ("rot_slow", _f),
                 ("qk_norm", _i), ("q_norm_dev", _vp), ("k_norm_dev", _vp), ("rot_half", _i), ("rot_scaling_kind", _i),
                 ("talk_dev", _vp), ("sink_dev", _vp), ("chunk", _i), ("v_mix", _i), ("v_mix_lambda", _f),
-                ("moe_router", _i), ("moe_gated", _i), ("moe_scale_input", _i), ("moe_shared_sg", _i)]
+                ("moe_router", _i), ("moe_gated", _i), ("moe_scale_input", _i), ("moe_shared_sg", _i),
+                ("w_in_bias_dev", _vp), ("window", _i), ("qk_head_norm", _i), ("diff_maps", _i), ("diff_lambda", _f), ("diff_init", _f),
+                ("decay_dev", _vp), ("post_norm_dev", _vp), ("post_norm2_dev", _vp),
+                ("side_gate_dev", _vp), ("side_proj_dev", _vp), ("side_norm_dev", _vp), ("side_col0", _i)]
 
 
 class TlHybridConfig(ctypes.Structure):
@@ -60,7 +63,7 @@ class TlHybridConfig(ctypes.Structure):
                 ("final_norm_offset", _f), ("head_dev", _vp),
                 ("embed_scale", _f), ("final_norm_kind", _i), ("final_norm_alpha", _f), ("final_norm_bias_dev", _vp),
                 ("page_size", _i), ("num_pages", _i), ("max_slots", _i), ("max_pages_per_seq", _i), ("max_rows", _i),
-                ("logit_scale", _f)]
+                ("logit_scale", _f), ("embed_norm_dev", _vp), ("side_embed_dev", _vp), ("side_cols", _i), ("side_dim", _i)]
 
 
 class TlHybridStats(ctypes.Structure):

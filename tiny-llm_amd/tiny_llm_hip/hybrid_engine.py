@@ -20,10 +20,10 @@ __all__ = ["HybridEngine"]
 
 _FF_ACT = {"gelu_erf": 0, "gelu_tanh": 1, "silu": 2, "relu2": 3}
 _MIX = {"attention": 0, "delta": 1, "linrec": 2, "latent": 3}
-_REC = {"channel": 0, "expgate": 1}
+_REC = {"channel": 0, "expgate": 1, "fixed": 2}
 _NORM = {"rms": 0, "dyt": 1}
 _FF_KIND = {"plain": 0, "gated": 1, "moe": 2}
-_BLOCK = {"sequential": 0, "parallel": 1, "postnorm": 2}
+_BLOCK = {"sequential": 0, "parallel": 1, "postnorm": 2, "sandwich": 3}
 _VMIX = {"none": 0, "first": 1, "blend": 2}
 _ROUTER = {"softmax": 0, "sigmoid": 1}
 
@@ -64,7 +64,7 @@ class HybridEngine:
             s.heads, s.kv_heads, s.dim, s.vdim, s.ff, s.ff_act = L.heads, L.kv_heads, L.dim, L.vdim, L.ff, _FF_ACT[L.ff_act]
             s.w_in_dev, s.w_out_dev, s.norm_dev, s.norm_offset = t["w_in"].data_ptr(), t["w_out"].data_ptr(), t["norm"].data_ptr(), cfg.norm_offset
             s.rot_dims, s.rot_base, s.scale = L.rot_dims, L.rot_base, L.scale
-            s.qk_unit_rms, s.sink, s.gated = int(L.qk_unit_rms), int(L.sink), int(L.gated)
+            s.qk_unit_rms, s.sink, s.gated = int(L.qk_unit_rms), int(L.sink), (2 if L.head_gate else 1) if L.gated else 0
             s.conv_taps, s.unit_eps = L.conv_taps, L.unit_eps
             if L.kind == "delta":
                 s.conv_dev, s.a_log_dev, s.dt_bias_dev, s.out_norm_dev = (t["conv"].data_ptr(), t["a_log"].data_ptr(),
@@ -82,11 +82,17 @@ class HybridEngine:
                 s.qk_norm, s.q_norm_dev, s.k_norm_dev, s.rot_half = int(L.qk_norm), ptr("q_norm"), ptr("k_norm"), int(L.rot_half)
                 s.talk_dev, s.sink_dev, s.chunk = ptr("talk"), ptr("sink"), L.chunk
                 s.v_mix, s.v_mix_lambda = _VMIX[L.v_mix], t.get("v_mix_lambda", 0.0)
-                if L.rot_scaling:
-                    s.rot_factor, s.rot_original, s.rot_fast, s.rot_slow = L.rot_scaling
-                    s.rot_scaling_kind = 1 if L.rot_scaling_kind == "wavelength" else 0
+                s.w_in_bias_dev, s.window, s.qk_head_norm = ptr("w_in_bias"), L.window, int(L.qk_head_norm)
+                if L.diff is not None:
+                    s.diff_maps, s.diff_lambda, s.diff_init = 1, t["diff_lambda"], L.diff
+            if L.kind in ("attention", "linrec") and L.rot_scaling:
+                s.rot_factor, s.rot_original, s.rot_fast, s.rot_slow = L.rot_scaling
+                s.rot_scaling_kind = 1 if L.rot_scaling_kind == "wavelength" else 0
+            s.post_norm_dev, s.post_norm2_dev = ptr("post_norm"), ptr("post_norm2")
+            s.side_gate_dev, s.side_proj_dev, s.side_norm_dev, s.side_col0 = ptr("side_gate"), ptr("side_proj"), ptr("side_norm"), i * cfg.side_dim
             if L.kind == "linrec":
-                s.rec_kind, s.gate_cap, s.tau, s.a_rank, s.out_norm_dev = _REC[L.rec_kind], L.gate_cap, L.tau, max(L.a_rank, 0), t["out_norm"].data_ptr()
+                s.rec_kind, s.gate_cap, s.tau, s.a_rank, s.out_norm_dev = _REC[L.rec_kind], L.gate_cap, L.tau, max(L.a_rank, 0), ptr("out_norm")
+                s.decay_dev, s.rot_half = ptr("decay"), int(L.rot_half)
                 s.a2_dev, s.a2_bias_dev, s.i_bias_dev, s.f_bias_dev = ptr("a2"), ptr("a2_bias"), ptr("i_bias"), ptr("f_bias")
             elif L.kind == "latent":
                 s.q_rank, s.kv_rank, s.rot_dim, s.kv_from = L.q_rank, L.kv_rank, L.rot_dim, L.kv_from
@@ -101,8 +107,11 @@ class HybridEngine:
         c.final_norm_bias_dev = w["final_norm_bias"].data_ptr() if "final_norm_bias" in w else None
         if cfg.loop:
             c.loop_start, c.loop_stop, c.loop_times = cfg.loop
-            c.loop_in_dev, c.loop_step_dev = w["loop_in"].data_ptr(), w["loop_step"].data_ptr()
+            c.loop_in_dev, c.loop_step_dev = (w["loop_in"].data_ptr() if "loop_in" in w else None), w["loop_step"].data_ptr()
         c.embed_dev, c.final_norm_dev, c.final_norm_offset, c.head_dev = w["embed"].data_ptr(), w["final_norm"].data_ptr(), cfg.norm_offset, w["head"].data_ptr()
+        c.embed_norm_dev = w["embed_norm"].data_ptr() if "embed_norm" in w else None
+        if cfg.side_dim:
+            c.side_embed_dev, c.side_cols, c.side_dim = w["side_embed"].data_ptr(), w["side_embed"].shape[1], cfg.side_dim
         c.page_size, c.num_pages, c.max_slots = self.page_size, int(num_pages), self.max_batch
         c.max_pages_per_seq = int(max_pages_per_seq if max_pages_per_seq is not None else num_pages)
         c.max_rows = self.max_prefill_rows

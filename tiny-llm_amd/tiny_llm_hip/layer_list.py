@@ -54,6 +54,21 @@ Lovulix -- x = embed[token]; per layer the norm sits on what a branch RETURNS an
         v <- (1 - vmix) v + vmix v_first (the first such layer's values of the same token); heads * sigmoid(W_g x); W_o.
     ff "moe": s = sigmoid(W_router x); the `top` largest s are taken; each contributes expert(s_e x) -- the score scales the expert's INPUT --
         with expert(u) = W_down (silu(W_gate u) * W_up u); plus a shared expert of the same form on x.
+
+Muduvik -- x = rms_norm(embed[token]) * embed.norm; every sublayer has a norm on both sides and a per-channel scale, and a layer ends with a
+per-layer token input:
+
+    x <- x + ls1 * norm1b(mixer(norm1 x));   x <- x + ls2 * norm2b(ff(norm2 x));   x <- x + rms_norm(W_sp (gelu_tanh(W_sg x) * e)) * side.norm
+    e = side.embed[token][i dim : (i + 1) dim] for layer i;   ff(h) = W_down (gelu_tanh(W_gate h) * W_up h);   norm: y / sqrt(mean y^2 + eps) * w
+
+    mixer "attention": differential attention.  q, k (with biases) hold two maps per head, [map 1 | map 2]; each map is RMS-normed over dim with one
+        [dim] weight, rotated on its first rot.dims dimensions (pairs (2i, 2i+1), frequencies rescaled by wavelength as in Lovulix), and is a softmax
+        attention of its own over keys j with 0 <= i - j < mask.size and the head group's shared values; o = a1 - lambda a2 with
+        lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, o / rms(o) * (1 - diff), times one sigmoid gate per head; W_o.
+    mixer "latent_attention": as Zefapel's without a rotated part and without a gate.
+    mixer "retention": q, k, v per head, q and k rotated (pairs (i, i + dims/2)), k * dim^-1/2;  S <- decay_h S + k v^T;  o = S^T q;
+        o / rms(o) * silu(W_g h); W_o.
+    loop {start, stop, times}: as Fonapel's, entered by x <- x + step[t] alone.
 """
 
 from __future__ import annotations
@@ -63,7 +78,7 @@ from typing import Any, Callable
 
 import torch
 
-__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "zefapel_config", "lovulix_config", "pack_layer_list"]
+__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "zefapel_config", "lovulix_config", "muduvik_config", "pack_layer_list"]
 
 
 @dataclass
@@ -119,6 +134,15 @@ class LayerSpec:
     moe_scale_input: bool = False   # the router's weight multiplies the expert's input
     moe_shared_sg: bool = True      # the shared expert is scaled by sigmoid of a scalar projection
     moe_correction: bool = True     # a selection-only correction vector (tensor mlp.correction)
+    # attention, further options (2)
+    bias: bool = False              # q, k, v carry biases (tensors mix.q.b / mix.k.b / mix.v.b)
+    window: int = 0                 # > 0: sliding window (a query sees itself and the window - 1 keys before it)
+    qk_head_norm: bool = False      # RMS norm per head (and map) over dim ahead of the rotation (tensors mix.q.norm / mix.k.norm [dim])
+    diff: float | None = None       # differential attention: two maps per head, lambda from mix.lq1 / lk1 / lq2 / lk2 and this constant
+    head_gate: bool = False         # gated: one gate number per head (tensor mix.g [heads, width])
+    # linrec "fixed": a constant decay per head
+    decay: tuple[float, ...] = ()
+    out_norm_weight: bool = True    # linrec: the read-out's unit-RMS norm has a weight (tensor mix.norm)
 
 
 @dataclass
@@ -137,6 +161,9 @@ class LayerListConfig:
     layer_scale: bool = False       # sequential block: per-channel vectors ls1 / ls2 on the branches
     embed_scale: float = 1.0
     logit_scale: float = 1.0
+    embed_norm: bool = False        # the embedding output passes the model's norm (tensor embed.norm)
+    loop_projection: bool = True    # a loop pass is entered through loop.in [width, 2 width]; False: only loop.step is added
+    side_dim: int = 0               # > 0: per-layer token input of this many columns a layer (tensors side.embed, <layer>.side.*)
     prefix: Callable[[int], str] = field(default=lambda i: f"l{i}.")
 
     @property
@@ -309,6 +336,91 @@ def _lovulix_tensor_shapes(cfg: LayerListConfig) -> dict[str, tuple[int, ...]]:
     return want
 
 
+def _rot(mc: dict) -> dict[str, Any]:
+    """rot {base, dims, scaling {factor, low, high, original}} -> LayerSpec fields (frequencies rescaled by wavelength)."""
+    rot = mc.get("rot") or {}
+    sc = None
+    if rot.get("scaling"):
+        g = rot["scaling"]
+        sc = (float(g["factor"]), float(g["original"]), float(g["high"]), float(g["low"]))
+    return dict(rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), rot_scaling=sc, rot_scaling_kind="wavelength")
+
+
+def muduvik_config(config: dict) -> LayerListConfig:
+    """config.json of a Muduvik checkpoint -> LayerListConfig.  Every size and every constant the file gives is read from it."""
+    for key in ("layers", "norm", "vocab", "width"):
+        if key not in config:
+            raise ValueError(f"config.json lacks {key!r}")
+    layers = []
+    for i, entry in enumerate(config["layers"]):
+        kind, mc, mlp = entry.get("type"), entry.get("mixer") or {}, entry.get("mlp")
+        ff: dict[str, Any] = {}
+        if mlp is not None:
+            if mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"layer {i}: unsupported mlp.kind={mlp.get('kind')!r} (dense only)")
+            ff = dict(ff=int(mlp["ff"]), ff_kind="gated", ff_act="gelu_tanh")
+        heads, dim, vdim = int(mc["heads"]), int(mc["dim"]), int(mc["vdim"])
+        if kind == "attention":
+            kv_heads = int(mc.get("kv_heads", heads))
+            if heads % kv_heads:
+                raise ValueError(f"layer {i}: {heads} heads do not form {kv_heads} equal groups")
+            layers.append(LayerSpec(kind="attention", heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=float(mc["scale"]), bias=True,
+                                    qk_head_norm=True, diff=float(mc["diff"]), window=int((mc.get("mask") or {}).get("size", 0)), gated=True,
+                                    head_gate=True, **_rot(mc), **ff))
+        elif kind == "latent_attention":
+            layers.append(LayerSpec(kind="latent", heads=heads, kv_heads=1, dim=dim, vdim=vdim, q_rank=int(mc["q_rank"]), kv_rank=int(mc["kv_rank"]),
+                                    scale=float(mc["scale"]), gated=False, **ff))
+        elif kind == "retention":
+            decay = tuple(float(d) for d in mc["decay"])
+            if len(decay) != heads:
+                raise ValueError(f"layer {i}: {len(decay)} decays for {heads} heads")
+            layers.append(LayerSpec(kind="linrec", rec_kind="fixed", heads=heads, kv_heads=heads, dim=dim, vdim=vdim, decay=decay, rot_half=True,
+                                    out_norm_weight=False, **_rot(mc), **ff))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+    loop = None
+    lp = config.get("loop")
+    if lp:
+        loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not (0 <= loop[0] < loop[1] <= len(layers)) or loop[2] < 1:
+            raise ValueError(f"loop {lp!r} does not fit {len(layers)} layers")
+    side = config.get("token_side") or {}
+    return LayerListConfig(family="Muduvik", width=int(config["width"]), vocab=int(config["vocab"]), norm_eps=float(config["norm"]["eps"]),
+                           residual_mult=1.0, layers=layers, norm_offset=0.0, loop=loop, block="sandwich", layer_scale=True, embed_norm=True,
+                           loop_projection=False, side_dim=int(side.get("dim", 0)))
+
+
+def _muduvik_tensor_shapes(cfg: LayerListConfig) -> dict[str, tuple[int, ...]]:
+    """Every tensor a Muduvik checkpoint must hold, with its shape."""
+    W, sd = cfg.width, cfg.side_dim
+    want: dict[str, tuple[int, ...]] = {"embed": (cfg.vocab, W), "embed.norm": (W,), "final.norm": (W,), "head": (cfg.vocab, W)}
+    if cfg.loop:
+        want["loop.step"] = (cfg.loop[2], W)
+    if sd:
+        want["side.embed"] = (cfg.vocab, sd * len(cfg.layers))
+    for i, L in enumerate(cfg.layers):
+        p, m = cfg.prefix(i), cfg.prefix(i) + "mix."
+        hv = L.heads * L.vdim
+        want.update({p + "norm1": (W,), p + "norm1b": (W,), p + "ls1": (W,), m + "o": (W, hv)})
+        if L.kind == "attention":
+            nq, nk, nv = 2 * L.heads * L.dim, 2 * L.kv_heads * L.dim, L.kv_heads * L.vdim
+            want.update({m + "q": (nq, W), m + "q.b": (nq,), m + "k": (nk, W), m + "k.b": (nk,), m + "v": (nv, W), m + "v.b": (nv,),
+                         m + "q.norm": (L.dim,), m + "k.norm": (L.dim,), m + "lq1": (L.dim,), m + "lk1": (L.dim,), m + "lq2": (L.dim,),
+                         m + "lk2": (L.dim,), m + "g": (L.heads, W)})
+        elif L.kind == "latent":
+            want.update({m + "dq": (L.q_rank, W), m + "dq.norm": (L.q_rank,), m + "uq": (L.heads * L.dim, L.q_rank), m + "dkv": (L.kv_rank, W),
+                         m + "dkv.norm": (L.kv_rank,), m + "uk": (L.heads * L.dim, L.kv_rank), m + "uv": (hv, L.kv_rank)})
+        else:
+            hd = L.heads * L.dim
+            want.update({m + "q": (hd, W), m + "k": (hd, W), m + "v": (hv, W), m + "g": (hv, W)})
+        if L.ff:
+            f = p + "mlp."
+            want.update({p + "norm2": (W,), p + "norm2b": (W,), p + "ls2": (W,), f + "gate": (L.ff, W), f + "up": (L.ff, W), f + "down": (W, L.ff)})
+        if sd:
+            want.update({p + "side.gate": (sd, W), p + "side.proj": (W, sd), p + "side.norm": (W,)})
+    return want
+
+
 def _norm_shapes(cfg: LayerListConfig, name: str) -> dict[str, tuple[int, ...]]:
     if cfg.norm_kind == "dyt":
         return {name: (cfg.width,), name + ".b": (cfg.width,), name + ".alpha": ()}
@@ -356,6 +468,7 @@ FAMILIES: dict[str, tuple[Callable[[dict], LayerListConfig], Callable[[LayerList
     "Fonapel": (fonapel_config, _fonapel_tensor_shapes),
     "Zefapel": (zefapel_config, _zefapel_tensor_shapes),
     "Lovulix": (lovulix_config, _lovulix_tensor_shapes),
+    "Muduvik": (muduvik_config, _muduvik_tensor_shapes),
 }
 
 
@@ -377,15 +490,20 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
 
     packed: dict[str, Any] = {"embed": mat("embed").contiguous(), "head": mat("head").contiguous(), "layers": []}
     norm(packed, "final_norm", "final.norm")
+    if cfg.embed_norm:
+        packed["embed_norm"] = vec("embed.norm")
+    if cfg.side_dim:
+        packed["side_embed"] = mat("side.embed").contiguous()
     if cfg.loop:
-        packed["loop_in"] = mat("loop.in").contiguous()
+        if cfg.loop_projection:
+            packed["loop_in"] = mat("loop.in").contiguous()
         packed["loop_step"] = vec("loop.step")
     for i, L in enumerate(cfg.layers):
         p = cfg.prefix(i)
         entry: dict[str, Any] = {}
         norm(entry, "norm", p + "norm1")
         if L.kind == "latent":
-            rows = [mat(p + "mix.dq")] + ([mat(p + "mix.dkv")] if L.kv_from < 0 else []) + [mat(p + "mix.g")]
+            rows = [mat(p + "mix.dq")] + ([mat(p + "mix.dkv")] if L.kv_from < 0 else []) + ([mat(p + "mix.g")] if L.gated else [])
             entry["dq_norm"], entry["uq"] = vec(p + "mix.dq.norm"), mat(p + "mix.uq").contiguous()
             if L.kv_from < 0:
                 entry["dkv_norm"] = vec(p + "mix.dkv.norm")
@@ -397,8 +515,14 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
             if L.kind != "attention" or L.gated:
                 rows.append(mat(p + "mix.g"))
         if L.kind == "attention":
-            if L.qk_norm:
+            if L.qk_norm or L.qk_head_norm:
                 entry["q_norm"], entry["k_norm"] = vec(p + "mix.q.norm"), vec(p + "mix.k.norm")
+            if L.bias:  # one vector over the mixer's rows of w_in: q | k | v biases, zeros behind them (the gate has none)
+                b = torch.cat([vec(p + "mix.q.b"), vec(p + "mix.k.b"), vec(p + "mix.v.b")])
+                entry["w_in_bias"] = torch.cat([b, torch.zeros(sum(r.shape[0] for r in rows) - b.numel(), device=device)]).contiguous()
+            if L.diff is not None:  # one number for the layer, from four [dim] vectors, in float32
+                t32 = lambda name: tensors[p + "mix." + name].to(torch.float32)
+                entry["diff_lambda"] = float(torch.exp((t32("lq1") * t32("lk1")).sum()) - torch.exp((t32("lq2") * t32("lk2")).sum()) + torch.tensor(L.diff, dtype=torch.float32))
             if L.talk:
                 entry["talk"] = vec(p + "mix.talk")
             if L.learned_sink:
@@ -410,8 +534,11 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
             entry["conv"] = torch.cat([vec(p + "mix.q.conv"), vec(p + "mix.k.conv"), vec(p + "mix.v.conv")], 0).contiguous()
             entry["a_log"], entry["dt_bias"], entry["out_norm"] = vec(p + "mix.A_log"), vec(p + "mix.dt_bias"), vec(p + "mix.norm")
         elif L.kind == "linrec":
-            entry["out_norm"] = vec(p + "mix.norm")
-            if L.rec_kind == "expgate":
+            if L.out_norm_weight:
+                entry["out_norm"] = vec(p + "mix.norm")
+            if L.rec_kind == "fixed":
+                entry["decay"] = torch.tensor(L.decay, dtype=torch.float32, device=device)
+            elif L.rec_kind == "expgate":
                 rows += [mat(p + "mix.i"), mat(p + "mix.f")]
                 entry["i_bias"], entry["f_bias"] = vec(p + "mix.i.b"), vec(p + "mix.f.b")
             else:
@@ -451,7 +578,13 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
                 rows, out = rows + ff_rows, out + ff_out
             else:
                 norm(entry, "norm2", p + "norm2")
+                if cfg.block == "sandwich":
+                    entry["post_norm2"] = vec(p + "norm2b")
                 entry["w_in2"], entry["w_out2"] = torch.cat(ff_rows, 0).contiguous(), torch.cat(ff_out, 1).contiguous()
+        if cfg.block == "sandwich":
+            entry["post_norm"] = vec(p + "norm1b")
+        if cfg.side_dim:
+            entry["side_gate"], entry["side_proj"], entry["side_norm"] = mat(p + "side.gate").contiguous(), mat(p + "side.proj").contiguous(), vec(p + "side.norm")
         if cfg.layer_scale:
             entry["ls1"] = vec(p + "ls1")
             if L.ff:
