@@ -789,3 +789,82 @@ def muduvik_forward(config, W, tokens, streams=None):
         if streams is not None:
             streams.append(x.copy())
     return rms_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+def make_muduvik_weights(config, seed=0):
+    """Random bf16-representable weights by tensor name (float32 arrays) for a Muduvik config dict."""
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    Wd, out = config["width"], {}
+
+    def mat(rows, cols, scale=None):
+        s = scale if scale is not None else cols ** -0.5
+        return (torch.randn(rows, cols, generator=gen) * s).to(torch.bfloat16).float().numpy()
+
+    def vec(n, scale=0.1, shift=0.0):
+        return (torch.randn(n, generator=gen) * scale + shift).to(torch.bfloat16).float().numpy()
+
+    n_layers, sd = len(config["layers"]), (config.get("token_side") or {}).get("dim", 0)
+    out["embed"], out["head"] = mat(config["vocab"], Wd, 1.0), mat(config["vocab"], Wd)
+    out["embed.norm"], out["final.norm"] = vec(Wd, 0.1, 1.0), vec(Wd, 0.1, 1.0)
+    if config.get("loop"):
+        out["loop.step"] = mat(config["loop"]["times"], Wd, 0.5)
+    if sd:
+        out["side.embed"] = mat(config["vocab"], sd * n_layers, 1.0)
+    for i, spec in enumerate(config["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", spec["mixer"]
+        H, D, V = mc["heads"], mc["dim"], mc["vdim"]
+        out[p + "norm1"], out[p + "norm1b"], out[p + "ls1"] = vec(Wd, 0.1, 1.0), vec(Wd, 0.1, 1.0), vec(Wd, 0.2, 0.6)
+        out[m + "o"] = mat(Wd, H * V)
+        if spec["type"] == "attention":
+            G = mc["kv_heads"]
+            out[m + "q"], out[m + "k"], out[m + "v"] = mat(2 * H * D, Wd), mat(2 * G * D, Wd), mat(G * V, Wd)
+            out[m + "q.b"], out[m + "k.b"], out[m + "v.b"] = vec(2 * H * D, 0.3), vec(2 * G * D, 0.3), vec(G * V, 0.3)
+            out[m + "q.norm"], out[m + "k.norm"] = vec(D, 0.2, 1.0), vec(D, 0.2, 1.0)
+            for name in ("lq1", "lk1", "lq2", "lk2"):
+                out[m + name] = vec(D, D ** -0.5)
+            out[m + "g"] = mat(H, Wd)
+        elif spec["type"] == "latent_attention":
+            out[m + "dq"], out[m + "dq.norm"], out[m + "uq"] = mat(mc["q_rank"], Wd), vec(mc["q_rank"], 0.1, 1.0), mat(H * D, mc["q_rank"])
+            out[m + "dkv"], out[m + "dkv.norm"] = mat(mc["kv_rank"], Wd), vec(mc["kv_rank"], 0.1, 1.0)
+            out[m + "uk"], out[m + "uv"] = mat(H * D, mc["kv_rank"]), mat(H * V, mc["kv_rank"])
+        else:
+            out[m + "q"], out[m + "k"], out[m + "v"], out[m + "g"] = mat(H * D, Wd), mat(H * D, Wd), mat(H * V, Wd), mat(H * V, Wd)
+        if spec.get("mlp"):
+            f, n = p + "mlp.", spec["mlp"]["ff"]
+            out[p + "norm2"], out[p + "norm2b"], out[p + "ls2"] = vec(Wd, 0.1, 1.0), vec(Wd, 0.1, 1.0), vec(Wd, 0.2, 0.6)
+            out[f + "gate"], out[f + "up"], out[f + "down"] = mat(n, Wd), mat(n, Wd), mat(Wd, n)
+        if sd:
+            out[p + "side.gate"], out[p + "side.proj"], out[p + "side.norm"] = mat(sd, Wd), mat(Wd, sd), vec(Wd, 0.1, 0.5)
+    return out
+
+
+def muduvik_attention(heads=4, kv_heads=2, dim=16, vdim=24, rot_dims=8, base=5000.0, scaling=(8.0, 1.0, 4.0, 64), scale=0.3, window=20, diff=0.4, ff=48):
+    rot = {"base": base, "dims": rot_dims}
+    if scaling:
+        rot["scaling"] = {"factor": scaling[0], "low": scaling[1], "high": scaling[2], "original": scaling[3]}
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot": rot, "scale": scale, "diff": diff}
+    if window:
+        mixer["mask"] = {"size": window}
+    return {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def muduvik_latent(heads=3, dim=16, vdim=24, q_rank=20, kv_rank=40, scale=0.2, ff=48):
+    return {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank, "scale": scale},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def muduvik_retention(heads=3, dim=16, vdim=24, rot_dims=8, base=3000.0, decay=None, ff=0):
+    decay = list(decay) if decay is not None else [1.0 - 2.0 ** (-3 - h) for h in range(heads)]
+    return {"type": "retention", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "rot": {"base": base, "dims": rot_dims}, "decay": decay},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def muduvik_config(layers, width=64, vocab=101, eps=1e-5, loop=None, side=8):
+    cfg = {"architecture": "Muduvik", "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    if side:
+        cfg["token_side"] = {"dim": side}
+    return cfg

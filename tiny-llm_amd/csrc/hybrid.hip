@@ -339,7 +339,11 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     const tl_hybrid_config &c = e->cfg;
     const StepShape sh = window_shape(sh0, x.window);
     const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
-    if (e->attn_rows_only || dk4 > 64 || vt_n > 16) {
+    // the two 64-wide tile templates serve widths that are multiples of 8 (whole 16-byte chunks); other widths beyond the 32-wide template
+    // take the row kernel, and float32 pages take the 16-tile value template for every width beyond 8 tiles
+    const bool whole_chunks = L.dim % 8 == 0 && L.vdim % 8 == 0 && v_row % 8 == 0;
+    const bool beyond_mid = dk4 > 32 || vt_n > 8;
+    if (e->attn_rows_only || dk4 > 64 || vt_n > 16 || (beyond_mid && !whole_chunks)) {
         hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(sh.rows, L.heads), dim3(64), (L.dim + 64) * sizeof(float), e->stream, e->qbuf, (const S *)kpool,
                            (const S *)vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim,
                            L.vdim, L.scale, L.sink, gate, ldg, (S *)out, ldo, v_row, x.window, x.vshare, x.gate_per_head, x.out32);
@@ -348,7 +352,7 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     }
     if (dk4 <= 16 && vt_n <= 4) return launch_attn_tile<D, 16, 4>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
     if (dk4 <= 32 && vt_n <= 8) return launch_attn_tile<D, 32, 8>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
-    if (vt_n <= 12) return launch_attn_tile<D, 64, 12>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);  // (a 192-wide latent beside a 64-wide rotated part)
+    if (vt_n <= 12 && sizeof(S) == 2) return launch_attn_tile<D, 64, 12>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);  // (a 192-wide latent beside a 64-wide rotated part)
     return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo, x);
 }
 
