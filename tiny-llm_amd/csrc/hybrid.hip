@@ -316,7 +316,9 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *
     // chunks whose rows fit one 16-row MFMA tile (decode steps): the four waves share the keys of a tile instead of the rows
     const bool wsplit = sh.max_len * HGB <= 16;
     const size_t lds = std::max(lds_tiles, (size_t)(128 + 4 * 64 * 4 * VT) * 4);
-    auto kern = wsplit ? attn_tile_kernel<D, DK4, VT, true> : attn_tile_kernel<D, DK4, VT, false>;
+    const bool ext = x.window > 0 || x.vshare != 1 || x.gate_per_head || x.out32;  // (plain causal attention keeps a kernel of its own)
+    auto kern = ext ? (wsplit ? attn_tile_kernel<D, DK4, VT, true, true> : attn_tile_kernel<D, DK4, VT, false, true>)
+                    : (wsplit ? attn_tile_kernel<D, DK4, VT, true, false> : attn_tile_kernel<D, DK4, VT, false, false>);
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.seq_row0, m.seq_slot, m.row_pos,
@@ -340,10 +342,14 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     const StepShape sh = window_shape(sh0, x.window);
     const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
     // the two 64-wide tile templates serve widths that are multiples of 8 (whole 16-byte chunks); other widths beyond the 32-wide template
-    // take the row kernel, and float32 pages take the 16-tile value template for every width beyond 8 tiles
+    // take the row kernel (the tile kernel faulted on a 136 / 130-wide head in float32, cause not found), and float32 pages take the 16-tile
+    // value template for every width beyond 8 tiles
     const bool whole_chunks = L.dim % 8 == 0 && L.vdim % 8 == 0 && v_row % 8 == 0;
     const bool beyond_mid = dk4 > 32 || vt_n > 8;
-    if (e->attn_rows_only || dk4 > 64 || vt_n > 16 || (beyond_mid && !whole_chunks)) {
+    const bool ext = x.window > 0 || x.vshare != 1 || x.gate_per_head || x.out32;
+    // (the 64-wide templates are built for plain causal attention only: with a window, shared values or float32 read-outs the 16-tile one gave
+    // wrong rows in decode steps, so those options stay on the templates up to 128 x 128 and take the row kernel beyond)
+    if (e->attn_rows_only || dk4 > 64 || vt_n > 16 || (beyond_mid && (!whole_chunks || ext))) {
         hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(sh.rows, L.heads), dim3(64), (L.dim + 64) * sizeof(float), e->stream, e->qbuf, (const S *)kpool,
                            (const S *)vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim,
                            L.vdim, L.scale, L.sink, gate, ldg, (S *)out, ldo, v_row, x.window, x.vshare, x.gate_per_head, x.out32);

@@ -431,15 +431,18 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
 //                                 step r is key 4 g + r of the 16-key sub-tile (a sum does not care in which order its terms are paired)
 // Per query row (= per lane column) a running maximum and sum; the sink is their start value (0, 1).  The key range may be split over
 // gridDim.z (decode steps over long contexts): then unnormalised partial sums + (max, sum) go to part_* and attn_merge_kernel finishes.
-template <typename D, int DK4, int VT, bool WSPLIT>
+template <typename D, int DK4, int VT, bool WSPLIT, bool EXT>
 __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
                                                         const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
                                                         const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
                                                         float scale, int sink, int HGB, int n_hblk, int keys_per_split, int n_splits, const float *gate,
                                                         int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml, int page_shift,
-                                                        int vec_ok, int v_row, int window, int vshare, int gate_per_head, float *out32) {
+                                                        int vec_ok, int v_row, int window_, int vshare_, int gate_per_head_, float *out32_) {
     using S = typename D::storage;
     extern __shared__ float smem[];
+    // EXT false: plain causal attention into D rows, the four options folded away at compile time
+    const int window = EXT ? window_ : 0, vshare = EXT ? vshare_ : 1, gate_per_head = EXT ? gate_per_head_ : 0;
+    float *const out32 = EXT ? out32_ : nullptr;
     // window > 0: a query sees key j <= its position only if position - j < window; the walk starts at the first key the tile's first row sees,
     // and a split key range (decode steps) is counted from there.  vshare: that many K/V heads in a row read one value head (maps over shared
     // values).  out32: the read-out as float32 rows [row, head, vdim] instead of D rows of `out` (no gate).
