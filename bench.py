@@ -845,9 +845,10 @@ def main() -> None:
     ap.add_argument("--layer-list", default=None, metavar="WIDTHS",
                     help="instead of the default workload: prefill / decode throughput of a layer-list model (Fonapel family) beside Qwen3 W4A16 at "
                          "equal layer sizes, e.g. 1024,2048,4096 (benches/layer_list_compare.py; one JSON line of its own, --prompt-len / --steps apply)")
-    ap.add_argument("--layer-list-family", default="Fonapel", choices=("Fonapel", "Zefapel", "Lovulix"),
+    ap.add_argument("--layer-list-family", default="Fonapel", choices=("Fonapel", "Zefapel", "Lovulix", "Muduvik"),
                     help="with --layer-list: the family measured.  Fonapel (default) stands beside Qwen3 W4A16; Zefapel stands beside Fonapel, its "
-                         "closest existing model, on the same engine; Lovulix beside Fonapel with attention layers only")
+                         "closest existing model, on the same engine; Lovulix beside Fonapel with attention layers only; Muduvik beside Zefapel with dense "
+                         "feed-forwards and beside Fonapel's attention layers")
     args = ap.parse_args()
     if args.layer_list is not None:
         from benches import layer_list_compare

@@ -18,6 +18,11 @@ all of them), a latent cache row of kv_rank + rot_dim per token.
 attention over the same paged K/V, one more norm per branch), at equal width, heads, head width and matrix elements a token multiplies:
 4 attention layers (16 heads at width 2048, a quarter of them K/V heads, scores mixed across heads, chunks of 8,192 positions, learned sinks,
 values blended from the second layer on) with 8 gated experts of W / 2 (2 taken) beside a shared one of W.
+
+`--layer-list-family Muduvik` measures the Muduvik family beside Zefapel with dense feed-forwards (the closest existing model: the same
+sequential block with layer scales, latent attention over the same 192-wide cache rows, a linear recurrence over 128 x 128 states, the
+same gated feed-forward of 2 W) and, for its attention layers, beside Fonapel's attention: 4 layers (retention, differential attention with
+a window of 4,096 positions, latent attention, differential attention), a per-layer token input of 256 columns.
 """
 
 from __future__ import annotations
@@ -61,6 +66,66 @@ def lovulix_costs(cfg: dict, ctx: int, dtype_bytes: int = 2) -> dict:
     return {"matrix_elems": fixed + sum(pe * top for pe, (top, _) in zip(per_expert, taken)), "head_elems": head, "attn_macs_per_pair": attn, "chunk": chunk,
             "decode_bytes": lambda b: (fixed + head + sum(pe * min(n, b * top) for pe, (top, n) in zip(per_expert, taken))) * dtype_bytes
             + b * seen * kv_per_tok * dtype_bytes}
+
+
+def muduvik_config(width: int, vocab: int = 32768, window: int = 4096, side: int = 256) -> dict:
+    heads = max(1, width // 128)
+    kv = max(1, heads // 4)
+    dense = {"kind": "dense", "ff": 2 * width}
+    rot = {"base": 5e5, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    attn = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "mask": {"size": window}, "rot": rot, "scale": 128 ** -0.5,
+                                           "diff": 0.6}, "mlp": dense}
+    ret = {"type": "retention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "rot": {"base": 1e6, "dims": 64},
+                                          "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(1, heads - 1)) for h in range(heads)]}, "mlp": dense}
+    lat = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "q_rank": max(64, width // 2), "kv_rank": 192, "scale": 128 ** -0.5},
+           "mlp": dense}
+    return {"architecture": "Muduvik", "layers": [ret, attn, lat, dict(attn)], "norm": {"eps": 1e-6}, "token_side": {"dim": side}, "vocab": vocab, "width": width}
+
+
+def muduvik_costs(cfg: dict, ctx: int, dtype_bytes: int = 2) -> dict:
+    """What the design needs: matrix elements a token multiplies, attention multiply-adds per (query, key) pair in the per-head form (two maps per
+    head in differential attention), the pairs a window leaves, and the bytes a decode step of b sequences streams: every matrix once, the keys
+    (two maps) and values inside the window, one latent row per cached token, the recurrent states read and written."""
+    W, sd = cfg["width"], (cfg.get("token_side") or {}).get("dim", 0)
+    fixed, state, windowed, causal = 0, 0, [], 0
+    kv_bytes = lambda c: 0
+    terms = []
+    for L in cfg["layers"]:
+        m, ff = L["mixer"], (L["mlp"] or {}).get("ff", 0)
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if L["type"] == "retention":
+            fixed += W * (2 * H * D + 2 * H * V) + H * V * W
+            state += H * D * V
+        elif L["type"] == "attention":
+            G, win = m["kv_heads"], (m.get("mask") or {}).get("size", 0)
+            fixed += W * (2 * H * D + 2 * G * D + G * V + H) + H * V * W
+            windowed.append((H * 2 * (D + V), win))
+            terms.append((G * (2 * D + V), win))
+        else:
+            C, Q = m["kv_rank"], m["q_rank"]
+            fixed += W * Q + Q * H * D + W * C + H * (D + V) * C + H * V * W
+            causal += H * (D + V)
+            terms.append((C, 0))
+        fixed += 3 * W * ff + 2 * W * sd
+    head = cfg["vocab"] * W
+
+    def attn_macs(n):  # multiply-adds of a causal prompt of n tokens
+        full = n * (n + 1) / 2
+        total = causal * full
+        for macs, win in windowed:
+            total += macs * (full if not win or win >= n else win * (win + 1) / 2 + (n - win) * win)
+        return total
+
+    return {"matrix_elems": fixed, "head_elems": head, "attn_macs": attn_macs,
+            "decode_bytes": lambda b: (fixed + head) * dtype_bytes + b * (sum(per * (min(ctx, win) if win else ctx) for per, win in terms) * dtype_bytes + 2 * state * 4)}
+
+
+def zefapel_dense_config(width: int, vocab: int = 32768) -> dict:
+    """Zefapel with the gated feed-forward of 2 W on every layer (no experts): the closest existing model to Muduvik, layer for layer."""
+    cfg = zefapel_config(width, vocab)
+    for L in cfg["layers"]:
+        L["mlp"] = {"kind": "dense", "ff": 2 * width}
+    return cfg
 
 
 def fonapel_config(width: int, layers: int = 4, vocab: int = 32768, order: str = "mixed") -> dict:
@@ -215,8 +280,12 @@ def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed
         page = 128
         pages = 4 * ((prompt_len + 3 * decode_steps) // page + 2)
         row = {"width": W, "prompt_len": prompt_len, "decode_steps": decode_steps}
-        new = ("zefapel", zefapel_config(W), zefapel_costs) if family == "Zefapel" else ("lovulix", lovulix_config(W), lovulix_costs)
-        for key, cfg, costs in (new, ("fonapel", fonapel_config(W, order="attention" if family == "Lovulix" else "mixed"), fonapel_costs)):
+        new = {"Zefapel": ("zefapel", zefapel_config(W), zefapel_costs), "Lovulix": ("lovulix", lovulix_config(W), lovulix_costs),
+               "Muduvik": ("muduvik", muduvik_config(W), muduvik_costs)}[family]
+        others = [("fonapel", fonapel_config(W, order="mixed" if family == "Zefapel" else "attention"), fonapel_costs)]
+        if family == "Muduvik":
+            others.insert(0, ("zefapel_dense", zefapel_dense_config(W), zefapel_costs))
+        for key, cfg, costs in [new] + others:
             model = synthetic_layer_list(cfg, seed=seed, device=device)
             eng = engine_for(model, dtype=torch.bfloat16, page_size=page, num_pages=pages, max_batch=4, max_pages_per_seq=pages // 4, max_prefill_rows=prompt_len)
             try:
@@ -226,11 +295,13 @@ def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed
             del model
             row[key] = summarize(got, costs(cfg, ctx), prompt_len)
             torch.cuda.empty_cache()
-        for leg in ("prefill", "decode_b1", "decode_b4"):
-            a, b = row[new[0]][leg]["roofline_fraction"], row["fonapel"][leg]["roofline_fraction"]
-            row.setdefault("times_as_far_from_roofline", {})[leg] = round(b / a, 2) if a > 0 else None
+        for other, _, _ in others:
+            for leg in ("prefill", "decode_b1", "decode_b4"):
+                a, b = row[new[0]][leg]["roofline_fraction"], row[other][leg]["roofline_fraction"]
+                name = "times_as_far_from_roofline" if other == others[0][0] else f"times_as_far_from_roofline_{other}"
+                row.setdefault(name, {})[leg] = round(b / a, 2) if a > 0 else None
         results.append(row)
-    return {"bench": "layer_list_compare", "family": family, "beside": "Fonapel", "dtype": "bf16", "data": "synthetic",
+    return {"bench": "layer_list_compare", "family": family, "beside": [o[0] for o in others] if len(others) > 1 else "Fonapel", "dtype": "bf16", "data": "synthetic",
             "roofline": {"hbm_bytes_per_s": HBM_BYTES_PER_S, "bf16_flops": BF16_FLOPS}, "results": results}
 
 
@@ -282,7 +353,8 @@ def run(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, d
 def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
     chunk = costs.get("chunk") or prompt_len  # a chunked mask: whole chunks and the prompt's last, partial one
     pairs = (prompt_len // chunk) * chunk * (chunk + 1) / 2 + (prompt_len % chunk) * (prompt_len % chunk + 1) / 2
-    flops = 2.0 * (costs["matrix_elems"] * prompt_len + costs["head_elems"]) + 2.0 * costs["attn_macs_per_pair"] * pairs
+    attn = costs["attn_macs"](prompt_len) if "attn_macs" in costs else costs["attn_macs_per_pair"] * pairs  # (a windowed design counts its own pairs)
+    flops = 2.0 * (costs["matrix_elems"] * prompt_len + costs["head_elems"]) + 2.0 * attn
     out = {"prefill": {"tokens_per_s": round(prompt_len / got["prefill_s"], 1), "ms": round(got["prefill_s"] * 1e3, 3), "tflops": round(flops / got["prefill_s"] / 1e12, 1),
                        "roofline_fraction": round(flops / got["prefill_s"] / BF16_FLOPS, 4)}}
     for b in (1, 4):
@@ -294,7 +366,7 @@ def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
 
 
 def main(widths, prompt_len=2048, decode_steps=64, family="Fonapel") -> None:
-    if family not in ("Fonapel", "Zefapel", "Lovulix"):
+    if family not in ("Fonapel", "Zefapel", "Lovulix", "Muduvik"):
         raise SystemExit(f"--layer-list-family: unknown family {family!r}")
     out = run(widths, prompt_len, decode_steps) if family == "Fonapel" else run_family_pair(widths, prompt_len, decode_steps, family=family)
     print(json.dumps(out), flush=True)

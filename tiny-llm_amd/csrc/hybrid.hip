@@ -497,7 +497,7 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
             const int M = attn_maps(L);
             hipLaunchKernelGGL((attn_prep_head_kernel<D>), dim3(rows, M * (H + G) + G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot, e->table_dev,
                                c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.rot_half, L.qk_head_norm, L.q_norm_dev, L.k_norm_dev, c.norm_eps,
-                               H, G, M, L.dim, L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+                               H, G, M, L.dim, L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool, L.w_in_bias_dev);
             TL_CHECK_LAUNCH("hybrid attention prep (per-head norm)");
             const float *gate = L.gated ? e->proj + (size_t)M * (H + G) * L.dim + (size_t)G * L.vdim : nullptr;
             AttnExtra x;
@@ -723,7 +723,9 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             const tl_hybrid_layer *Nx = (ri + 1 < e->runs.size() && !e->runs[ri + 1].enters_pass) ? &e->layers[e->runs[ri + 1].layer] : nullptr;
             const bool side = L.side_gate_dev != nullptr;
             const int threads = rows < 64 ? 1024 : 256;
-            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, L.w_in_bias_dev ? 2 : 0, 1.f, L.w_in_bias_dev, 0, st));
+            // (biases: the per-head preparation of an attention layer adds them where it reads q, k and v; any other mixer gets them with the product)
+            const bool prep_adds_bias = L.kind == TL_MIX_ATTENTION && (L.diff_maps || L.qk_head_norm || L.window > 0 || L.gated == 2);
+            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, L.w_in_bias_dev && !prep_adds_bias ? 2 : 0, 1.f, L.w_in_bias_dev, 0, st));
             HY_TRY(mixer_t<D>(e, ri, m, sh, nmix, HV));
             HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->y, W, rows, W, HV, 0, 1.f, nullptr, 0, st));
             {

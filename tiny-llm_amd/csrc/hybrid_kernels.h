@@ -30,7 +30,10 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 __device__ __forceinline__ float act_f(float z, int kind) {
     if (kind == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f));
-    if (kind == 1) return 0.5f * z * (1.f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+    if (kind == 1) {  // 0.5 z (1 + tanh u) = z / (1 + exp(-2 u)), u = sqrt(2/pi) (z + 0.044715 z^3): one exponential instead of tanhf
+        const float u = 0.79788456080286535588f * (z + 0.044715f * z * z * z);
+        return z / (1.f + expf(-2.f * u));
+    }
     return silu_f(z);
 }
 
@@ -42,17 +45,32 @@ __global__ void embed_kernel(const int32_t *tokens, const typename D::storage *e
     const int t = blockIdx.x;
     int tok = tokens[t];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
-    float inv = 1.f;
+    float inv = 1.f, keep[16];  // (the row's first 16 elements a thread stay in registers between the two passes)
     if (nw) {
         float ss = 0.f;
-        for (int c = threadIdx.x; c < width; c += blockDim.x) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * blockDim.x;
+            keep[i] = c < width ? ld<D>(embed, (size_t)tok * width + c) * scale : 0.f;
+            ss += keep[i] * keep[i];
+        }
+        for (int c = threadIdx.x + 16 * blockDim.x; c < width; c += blockDim.x) {
             const float v = ld<D>(embed, (size_t)tok * width + c) * scale;
             ss += v * v;
         }
         ss = block_sum(ss, red);
         inv = 1.f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * blockDim.x;
+            if (c < width) {
+                const float v = keep[i] * inv * (noffset + nw[c]);
+                x0[(size_t)t * width + c] = v;
+                x[(size_t)t * width + c] = v;
+            }
+        }
     }
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    for (int c = threadIdx.x + (nw ? 16 * blockDim.x : 0); c < width; c += blockDim.x) {
         float v = ld<D>(embed, (size_t)tok * width + c) * scale;
         if (nw) v = v * inv * (noffset + nw[c]);
         x0[(size_t)t * width + c] = v;
@@ -727,25 +745,30 @@ template <typename D>
 __global__ __launch_bounds__(64) void attn_prep_head_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
                                                             const int32_t *block_table, int max_pages, int page_size, const float *inv_freq, int rot_dims,
                                                             int rot_half, int head_norm, const float *qw, const float *kw, float eps, int H, int G, int M, int dim,
-                                                            int vdim, float *qbuf, typename D::storage *kpool, typename D::storage *vpool) {
+                                                            int vdim, float *qbuf, typename D::storage *kpool, typename D::storage *vpool, const float *bias) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const int pos = row_pos[t], slot = seq_slot[row_seq[t]];
     const int page = block_table[(size_t)slot * max_pages + pos / page_size], in_page = pos % page_size;
     const int HM = H * M, GM = G * M;
     if (hh >= HM + GM) {  // a value head: copy
         const int g = hh - HM - GM;
-        const float *src = proj + (size_t)t * ldp + (size_t)(HM + GM) * dim + (size_t)g * vdim;
+        const size_t col = (size_t)(HM + GM) * dim + (size_t)g * vdim;
+        const float *src = proj + (size_t)t * ldp + col;
         typename D::storage *dst = vpool + (((size_t)page * G + g) * page_size + in_page) * vdim;
-        for (int c = lane; c < vdim; c += 64) dst[c] = D::from_float(src[c]);
+        for (int c = lane; c < vdim; c += 64) dst[c] = D::from_float(src[c] + (bias ? bias[col + c] : 0.f));
         return;
     }
     const bool is_q = hh < HM;
     const float *src = proj + (size_t)t * ldp + (size_t)hh * dim;
+    const float *bs = bias ? bias + (size_t)hh * dim : nullptr;  // bias (NULL: none): the projection's, over the columns of proj, added here
     const float *w = head_norm ? (is_q ? qw : kw) : nullptr;
     float inv = 1.f;
     if (head_norm) {
         float ss = 0.f;
-        for (int c = lane; c < dim; c += 64) ss += src[c] * src[c];
+        for (int c = lane; c < dim; c += 64) {
+            const float v = src[c] + (bs ? bs[c] : 0.f);
+            ss += v * v;
+        }
         ss = wave_sum(ss);
         inv = 1.f / sqrtf(ss / (float)dim + eps);
     }
@@ -761,9 +784,9 @@ __global__ __launch_bounds__(64) void attn_prep_head_kernel(const float *proj, i
         int c0, c1 = -1;
         if (u < half) c0 = rot_half ? u : 2 * u, c1 = rot_half ? u + half : 2 * u + 1;
         else c0 = u + half;
-        float a = src[c0] * inv * (w ? w[c0] : 1.f), b2 = 0.f;
+        float a = (src[c0] + (bs ? bs[c0] : 0.f)) * inv * (w ? w[c0] : 1.f), b2 = 0.f;
         if (c1 >= 0) {
-            b2 = src[c1] * inv * (w ? w[c1] : 1.f);
+            b2 = (src[c1] + (bs ? bs[c1] : 0.f)) * inv * (w ? w[c1] : 1.f);
             float sn, cs;
             sincosf((float)pos * inv_freq[u], &sn, &cs);
             const float na = a * cs - b2 * sn, nb = b2 * cs + a * sn;

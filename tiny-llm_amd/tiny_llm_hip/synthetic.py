@@ -140,7 +140,7 @@ def synthetic_layer_list(config: dict, seed: int = 0, device: str = "cuda", dtyp
         if getattr(L, "a_rank", 0) < 0:
             L.a_rank = 16
     # vectors that multiply (norm weights applied as they are, layer scales) are drawn around 1, biases that open a gate around their shift
-    around_one = ("mix.norm", ".alpha") + ((".norm1", ".norm2", "final.norm", "dq.norm", "dkv.norm", "mix.q.norm", "mix.k.norm", ".ls1", ".ls2") if cfg.norm_offset == 0.0 else ())
+    around_one = ("mix.norm", ".alpha") + ((".norm1", ".norm2", "final.norm", "dq.norm", "dkv.norm", "mix.q.norm", "mix.k.norm", ".ls1", ".ls2", ".norm1b", ".norm2b", "embed.norm", "side.norm") if cfg.norm_offset == 0.0 else ())
     shifts = {"mix.f.b": 3.0, "mix.a2.b": 2.0}
     for name, shape in tensor_shapes(cfg).items():
         shift = 1.0 if name.endswith(around_one) else next((v for k, v in shifts.items() if name.endswith(k)), 0.0)
