@@ -72,9 +72,9 @@ def muduvik_config(width: int, vocab: int = 32768, window: int = 4096, side: int
     heads = max(1, width // 128)
     kv = max(1, heads // 4)
     dense = {"kind": "dense", "ff": 2 * width}
-    rot = {"base": 5e5, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    rot = {"base": 1e6, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
     attn = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "mask": {"size": window}, "rot": rot, "scale": 128 ** -0.5,
-                                           "diff": 0.6}, "mlp": dense}
+                                           "diff": 0.5}, "mlp": dense}
     ret = {"type": "retention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "rot": {"base": 1e6, "dims": 64},
                                           "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(1, heads - 1)) for h in range(heads)]}, "mlp": dense}
     lat = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "q_rank": max(64, width // 2), "kv_rank": 192, "scale": 128 ** -0.5},

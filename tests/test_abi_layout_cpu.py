@@ -35,11 +35,24 @@ def c_fields(header: str, struct: str) -> list[str]:
     return names
 
 
+HYBRID_PAIRS = {"tl_hybrid_layer": "TlHybridLayer", "tl_hybrid_config": "TlHybridConfig", "tl_hybrid_stats": "TlHybridStats"}
+
+
 def test_ctypes_structs_match_the_c_layout(tmp_path):
     import tiny_llm_ext_hip as ext
 
-    header = (ROOT / "include" / "tinyllm_engine.h").read_text()
-    lines = ["#include <stdio.h>", "#include <stddef.h>", '#include "tinyllm_engine.h"', "int main(void) {"]
+    _check(tmp_path, ext, "tinyllm_engine.h", PAIRS)
+
+
+def test_ctypes_structs_of_the_layer_list_engine_match_the_c_layout(tmp_path):
+    import tiny_llm_ext_hybrid as ext
+
+    _check(tmp_path, ext, "tinyllm_hybrid.h", HYBRID_PAIRS)
+
+
+def _check(tmp_path, ext, header_name, PAIRS):
+    header = (ROOT / "include" / header_name).read_text()
+    lines = ["#include <stdio.h>", "#include <stddef.h>", f'#include "{header_name}"', "int main(void) {"]
     for struct in PAIRS:
         lines.append(f'    printf("{struct} size %zu\\n", sizeof({struct}));')
         for f in c_fields(header, struct):

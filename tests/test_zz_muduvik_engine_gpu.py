@@ -82,9 +82,9 @@ def test_each_mechanism_alone(layer, dtype):
         engine.close()
 
 
-@pytest.mark.parametrize("side,loop", [(0, None), (5, None), (8, (0, 1, 1)), (3, (0, 3, 3)), (0, (1, 3, 2)), (16, (2, 3, 4))])
+@pytest.mark.parametrize("side,loop", [(0, None), (5, None), (8, (0, 1, 1)), (3, (0, 3, 3)), (0, (1, 3, 2)), (12, (2, 3, 4))])
 def test_token_input_and_loops(side, loop):
-    """No token input, inputs of 3 to 16 columns a layer; no loop, a loop of one pass, the whole model looped, loops that start behind the
+    """No token input, inputs of 3 to 12 columns a layer; no loop, a loop of one pass, the whole model looped, loops that start behind the
     first layer and end with the last: every pass has its own pages and state and its own offset."""
     config = O.muduvik_config([O.muduvik_retention(), O.muduvik_attention(window=9), O.muduvik_latent()], side=side, loop=loop)
     W = O.make_muduvik_weights(config, seed=40)
